@@ -1,0 +1,43 @@
+// Library identity, status strings and the option store of libe2h_quant.so.
+#include <string.h>
+
+#include "e2h_common.h"
+
+namespace e2h {
+Options &options() {
+  static Options o = {0, 0, 0};
+  return o;
+}
+}  // namespace e2h
+
+extern "C" int e2h_abi_version(void) { return E2H_ABI_VERSION; }
+
+extern "C" const char *e2h_status_string(int status) {
+  switch (status) {
+    case E2H_OK: return "ok";
+    case E2H_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case E2H_ERR_BAD_SHAPE: return "unsupported shape (m, n, k)";
+    case E2H_ERR_BAD_GROUPSIZE: return "groupsize must be one of 32, 64, 128, 256 and divide k";
+    case E2H_ERR_BAD_INNER_K_TILES: return "inner_k_tiles must be one of 2, 4, 8 and 16*inner_k_tiles must divide k";
+    case E2H_ERR_MISALIGNED: return "pointer not aligned as required";
+    case E2H_ERR_LAUNCH: return "HIP kernel launch failed";
+    case E2H_ERR_NO_DEVICE: return "no gfx950 device";
+    case E2H_ERR_BAD_OPTION: return "unknown option or value out of range";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int e2h_set_option(const char *name, int value) {
+  if (!name) return E2H_ERR_NULL_POINTER;
+  e2h::Options &o = e2h::options();
+  if (!strcmp(name, "int4_rows_per_wave") || !strcmp(name, "int8_rows_per_wave")) {
+    if (value != 0 && value != 16 && value != 32 && value != 64) return E2H_ERR_BAD_OPTION;
+    (name[3] == '4' ? o.int4_rows_per_wave : o.int8_rows_per_wave) = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "x_transpose")) {
+    o.x_transpose = value;
+    return E2H_OK;
+  }
+  return E2H_ERR_BAD_OPTION;
+}

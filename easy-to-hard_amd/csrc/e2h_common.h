@@ -1,0 +1,47 @@
+// Shared device/host helpers for the gfx950 kernels behind include/e2h_quant.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/e2h_quant.h"
+
+namespace e2h {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWaveSize = 64;
+
+// ---- bfloat16 <-> float32 (bit exact, round to nearest even; NaN inputs are not expected) --------
+
+__host__ __device__ inline float bf16_to_f32(uint16_t b) {
+  uint32_t u = static_cast<uint32_t>(b) << 16;
+  return __builtin_bit_cast(float, u);
+}
+
+__host__ __device__ inline uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+// float32 value rounded to the nearest bfloat16, kept as float32
+__host__ __device__ inline float bf16_round(float f) { return bf16_to_f32(f32_to_bf16_rne(f)); }
+
+// ---- option store (set through e2h_set_option) --------------------------------------------------
+
+struct Options {
+  int int4_rows_per_wave;  // 0 = heuristic, else 16/32/64
+  int int8_rows_per_wave;  // 0 = heuristic, else 16/32/64
+  int x_transpose;         // 0 = heuristic
+};
+Options &options();
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? E2H_OK : E2H_ERR_LAUNCH; }
+
+}  // namespace e2h

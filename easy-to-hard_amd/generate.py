@@ -1,0 +1,92 @@
+"""Batched greedy decoding and reward scoring on top of model.Transformer (harness for the decode configs).
+
+Follows the control flow of the reference's inference_generate.py (`prefill` :98-107, `decode_one_token`
+:110-120, `decode_n_tokens` :123-157, `generate` :164-221) with greedy argmax in place of sampling, and of
+inference_reward.py `model_score` (:67-91).  The decode step can be captured once into a HIP graph and
+replayed per token: every kernel of this package enqueues on the current stream with a launch geometry
+that depends on shapes only.
+"""
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+
+def greedy_token(logits: Tensor) -> Tensor:
+    """argmax over the vocabulary of the last position, in float32 -> [B, 1] int64."""
+    return torch.argmax(logits[:, -1].float(), dim=-1, keepdim=True)
+
+
+@torch.no_grad()
+def prefill(model, x: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None) -> Tensor:
+    return greedy_token(model(x, input_pos, left_pad_mask_pos))
+
+
+@torch.no_grad()
+def decode_one_token(model, cur_token: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None) -> Tensor:
+    assert input_pos.shape[-1] == 1
+    return greedy_token(model(cur_token, input_pos, left_pad_mask_pos))
+
+
+class GraphedDecodeStep:
+    """One decode step captured into a HIP graph; `step(token, pos)` copies the inputs into the static
+    buffers, replays the graph and returns the static output buffer ([B, 1] next tokens)."""
+
+    def __init__(self, model, batch_size: int, device, left_pad_mask_pos: Optional[Tensor] = None, warmup: int = 2):
+        self.model = model
+        self.cur_token = torch.zeros((batch_size, 1), dtype=torch.int64, device=device)
+        self.input_pos = torch.zeros((1,), dtype=torch.int64, device=device)
+        self.left_pad = left_pad_mask_pos
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side):
+            for _ in range(warmup):
+                decode_one_token(model, self.cur_token, self.input_pos, self.left_pad)
+        torch.cuda.current_stream(device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.next_token = decode_one_token(model, self.cur_token, self.input_pos, self.left_pad)
+
+    def step(self, cur_token: Tensor, input_pos: Tensor) -> Tensor:
+        self.cur_token.copy_(cur_token)
+        self.input_pos.copy_(input_pos)
+        self.graph.replay()
+        return self.next_token
+
+
+@torch.no_grad()
+def generate(model, prompt: Tensor, max_new_tokens: int, use_graph: bool = True,
+             left_pad_mask_pos: Optional[Tensor] = None, stepper: Optional[GraphedDecodeStep] = None) -> Tensor:
+    """prompt [B, T] int64 on the GPU -> [B, T + max_new_tokens] (prompt followed by greedy tokens)."""
+    bsz, t = prompt.shape
+    total = t + max_new_tokens
+    device = prompt.device
+    model.setup_caches(max_batch_size=bsz, max_seq_length=min(total, model.config.block_size))
+    seq = torch.empty((bsz, total), dtype=prompt.dtype, device=device)
+    seq[:, :t] = prompt
+    input_pos = torch.arange(0, t, device=device)
+    cur = prefill(model, prompt, input_pos, left_pad_mask_pos)
+    seq[:, t] = cur[:, 0]
+    if max_new_tokens > 1:
+        if use_graph and stepper is None:
+            stepper = GraphedDecodeStep(model, bsz, device, left_pad_mask_pos)
+            # the capture warm-up wrote garbage K/V at position 0 of the cache: recompute the prompt
+            cur = prefill(model, prompt, input_pos, left_pad_mask_pos)
+        pos = torch.tensor([t], device=device, dtype=torch.int64)
+        for i in range(1, max_new_tokens):
+            if stepper is not None:
+                cur = stepper.step(cur, pos).clone()
+            else:
+                cur = decode_one_token(model, cur, pos, left_pad_mask_pos)
+            seq[:, t + i] = cur[:, 0]
+            pos += 1
+    return seq
+
+
+@torch.no_grad()
+def model_score(reward_model, prompt: Tensor, max_seq_len: Optional[int] = None) -> Tensor:
+    """Per-token rewards [B, T] of a RewardModel on a fully causal pass without KV cache."""
+    bsz, t = prompt.shape
+    reward_model.backbone.setup_caches(max_batch_size=bsz, max_seq_length=max_seq_len or t, kv_cache=False)
+    return reward_model(prompt)

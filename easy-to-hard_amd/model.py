@@ -1,0 +1,273 @@
+"""Minimal Llama-family decoder that hosts the quantized linears (harness for the decode / reward configs).
+
+It reproduces the forward semantics and the state-dict key names of the reference's models/model.py
+(Transformer :132-252, TransformerBlock :255-283, Attention :286-349, FeedForward :352-360, RMSNorm
+:363-386, RoPE cache :389-412, KVCache :112-129, configs :78-109) so that a QuantHandler from
+quantize.py can swap its nn.Linear children and a reference checkpoint loads key for key.  Attention,
+normalisation and RoPE are stock PyTorch ops; only the linears are this package's kernels.
+"""
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+from .quantize import find_multiple
+
+
+@dataclass
+class ModelArgs:
+    """reference models/model.py:42-75."""
+
+    block_size: int = 2048
+    vocab_size: int = 32000
+    n_layer: int = 32
+    n_head: int = 32
+    dim: int = 4096
+    intermediate_size: Optional[int] = None
+    n_local_heads: int = -1
+    head_dim: int = 64
+    rope_base: float = 10000
+    norm_eps: float = 1e-5
+
+    def __post_init__(self):
+        if self.n_local_heads == -1:
+            self.n_local_heads = self.n_head
+        if self.intermediate_size is None:
+            self.intermediate_size = find_multiple(int(2 * (4 * self.dim) / 3), 256)
+        self.head_dim = self.dim // self.n_head
+
+    @classmethod
+    def from_name(cls, name: str):
+        if name in transformer_configs:
+            return cls(**transformer_configs[name])
+        matches = [c for c in transformer_configs if c in str(name).upper() or c in str(name)]
+        assert len(matches) >= 1, name
+        return cls(**transformer_configs[matches[0]])
+
+
+# reference models/model.py:78-109 (shapes only), plus small shapes for tests
+transformer_configs = {
+    "CodeLlama-7b-Python-hf": dict(block_size=16384, vocab_size=32000, n_layer=32, dim=4096, rope_base=1000000),
+    "llemma-7b": dict(block_size=4096, n_layer=32, n_head=32, dim=4096),
+    "deepseek-math-7b": dict(block_size=4096, vocab_size=102400, n_layer=30, n_head=32, dim=4096,
+                             intermediate_size=11008, rope_base=10000, norm_eps=1e-6),
+    "7B": dict(n_layer=32, n_head=32, dim=4096),
+    "13B": dict(n_layer=40, n_head=40, dim=5120),
+    "30B": dict(n_layer=60, n_head=52, dim=6656),
+    "34B": dict(block_size=4096, n_layer=48, n_head=64, dim=8192, vocab_size=32000, n_local_heads=8,
+                intermediate_size=22016, rope_base=1000000),
+    "70B": dict(n_layer=80, n_head=64, dim=8192, n_local_heads=8, intermediate_size=28672),
+    "tiny-test": dict(block_size=256, vocab_size=512, n_layer=2, n_head=4, dim=256, intermediate_size=512),
+    "tiny-gqa-test": dict(block_size=256, vocab_size=512, n_layer=2, n_head=8, n_local_heads=2, dim=512,
+                          intermediate_size=1024),
+}
+
+
+class KVCache(nn.Module):
+    """bf16 [B, H_kv, S_max, D] key and value caches written at `input_pos` (reference :112-129)."""
+
+    def __init__(self, max_batch_size, max_seq_length, n_heads, head_dim, dtype=torch.bfloat16, device=None):
+        super().__init__()
+        shape = (max_batch_size, n_heads, max_seq_length, head_dim)
+        self.register_buffer("k_cache", torch.zeros(shape, dtype=dtype, device=device))
+        self.register_buffer("v_cache", torch.zeros(shape, dtype=dtype, device=device))
+
+    def update(self, input_pos, k_val, v_val):
+        assert input_pos.shape[0] == k_val.shape[2]
+        bsz = k_val.size(0)
+        self.k_cache[:bsz].index_copy_(2, input_pos, k_val)
+        self.v_cache[:bsz].index_copy_(2, input_pos, v_val)
+        return self.k_cache[:bsz], self.v_cache[:bsz]
+
+
+class RMSNorm(nn.Module):
+    """x * rsqrt(mean(x^2) + eps) in float32, cast back, times weight (reference :363-377)."""
+
+    def __init__(self, dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: Tensor) -> Tensor:
+        xf = x.float()
+        normed = xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + self.eps)
+        return normed.to(dtype=x.dtype) * self.weight
+
+
+def precompute_freqs_cis(seq_len: int, n_elem: int, base: float = 10000, device=None) -> Tensor:
+    """[seq_len, n_elem/2, 2] (cos, sin) table stored in bfloat16 (reference :389-397)."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, n_elem, 2, device=device)[: n_elem // 2].float() / n_elem))
+    angles = torch.outer(torch.arange(seq_len, device=device), inv_freq)
+    return torch.stack([torch.cos(angles), torch.sin(angles)], dim=-1).to(dtype=torch.bfloat16)
+
+
+def apply_rotary_emb(x: Tensor, freqs_cis: Tensor) -> Tensor:
+    """Rotate interleaved pairs (x[2i], x[2i+1]) by the cached angle; float32 math (reference :400-412).
+
+    x [B, S, H, D], freqs_cis [S, D/2, 2]."""
+    pairs = x.float().reshape(*x.shape[:-1], -1, 2)
+    fc = freqs_cis.view(1, pairs.size(1), 1, pairs.size(3), 2)
+    re = pairs[..., 0] * fc[..., 0] - pairs[..., 1] * fc[..., 1]
+    im = pairs[..., 1] * fc[..., 0] + pairs[..., 0] * fc[..., 1]
+    return torch.stack([re, im], dim=-1).flatten(3).type_as(x)
+
+
+class Attention(nn.Module):
+    def __init__(self, config: ModelArgs):
+        super().__init__()
+        assert config.dim % config.n_head == 0
+        total_head_dim = (config.n_head + 2 * config.n_local_heads) * config.head_dim
+        self.wqkv = nn.Linear(config.dim, total_head_dim, bias=False)  # rows ordered [q | k | v]
+        self.wo = nn.Linear(config.dim, config.dim, bias=False)
+        self.kv_cache = None
+        self.n_head = config.n_head
+        self.head_dim = config.head_dim
+        self.n_local_heads = config.n_local_heads
+        self.dim = config.dim
+        self._register_load_state_dict_pre_hook(self._fuse_qkv_hook)
+
+    @staticmethod
+    def _fuse_qkv_hook(state_dict, prefix, *args):
+        # checkpoints with separate wq/wk/wv are fused on load (reference :303-308)
+        if prefix + "wq.weight" in state_dict:
+            parts = [state_dict.pop(prefix + n + ".weight") for n in ("wq", "wk", "wv")]
+            state_dict[prefix + "wqkv.weight"] = torch.cat(parts)
+
+    def forward(self, x: Tensor, freqs_cis: Tensor, mask: Optional[Tensor], input_pos: Optional[Tensor] = None,
+                fully_causal: bool = False) -> Tensor:
+        bsz, seqlen, _ = x.shape
+        kv_size = self.n_local_heads * self.head_dim
+        q, k, v = self.wqkv(x).split([self.dim, kv_size, kv_size], dim=-1)
+        q = apply_rotary_emb(q.view(bsz, seqlen, self.n_head, self.head_dim), freqs_cis).transpose(1, 2)
+        k = apply_rotary_emb(k.view(bsz, seqlen, self.n_local_heads, self.head_dim), freqs_cis).transpose(1, 2)
+        v = v.view(bsz, seqlen, self.n_local_heads, self.head_dim).transpose(1, 2)
+        if not fully_causal:
+            k, v = self.kv_cache.update(input_pos, k, v)
+        rep = self.n_head // self.n_local_heads
+        if rep > 1:
+            k = k.repeat_interleave(rep, dim=1)
+            v = v.repeat_interleave(rep, dim=1)
+        if fully_causal and q.size(2) == k.size(2):
+            y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        else:
+            y = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+        y = y.transpose(1, 2).contiguous().view(bsz, seqlen, self.dim)
+        return self.wo(y)
+
+
+class FeedForward(nn.Module):
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.w1 = nn.Linear(config.dim, config.intermediate_size, bias=False)
+        self.w3 = nn.Linear(config.dim, config.intermediate_size, bias=False)
+        self.w2 = nn.Linear(config.intermediate_size, config.dim, bias=False)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+
+
+class TransformerBlock(nn.Module):
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.attention = Attention(config)
+        self.feed_forward = FeedForward(config)
+        self.ffn_norm = RMSNorm(config.dim, config.norm_eps)
+        self.attention_norm = RMSNorm(config.dim, config.norm_eps)
+
+    def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Optional[Tensor], fully_causal: bool = False) -> Tensor:
+        h = x + self.attention(self.attention_norm(x), freqs_cis, mask, input_pos, fully_causal)
+        return h + self.feed_forward(self.ffn_norm(h))
+
+
+class Transformer(nn.Module):
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.config = config
+        self.tok_embeddings = nn.Embedding(config.vocab_size, config.dim)
+        self.layers = nn.ModuleList(TransformerBlock(config) for _ in range(config.n_layer))
+        self.norm = RMSNorm(config.dim, eps=config.norm_eps)
+        self.output = nn.Linear(config.dim, config.vocab_size, bias=False)
+        self.freqs_cis: Optional[Tensor] = None
+        self.causal_mask: Optional[Tensor] = None
+        self.self_mask: Optional[Tensor] = None
+        self.max_batch_size = -1
+        self.max_seq_length = -1
+        self.kv_cache_enabled = False
+
+    @classmethod
+    def from_name(cls, name: str):
+        return cls(ModelArgs.from_name(name))
+
+    def setup_caches(self, max_batch_size, max_seq_length, kv_cache=True):
+        """reference :172-210.  Caches are created on the device of the embedding table."""
+        if self.max_seq_length >= max_seq_length and self.max_batch_size >= max_batch_size:
+            if self.kv_cache_enabled or not kv_cache:
+                return
+        device = self.tok_embeddings.weight.device
+        cfg = self.config
+        max_seq_length = find_multiple(max_seq_length, 8)
+        self.max_seq_length = max_seq_length
+        self.max_batch_size = max_batch_size
+        for blk in self.layers:
+            blk.attention.kv_cache = (
+                KVCache(max_batch_size, max_seq_length, cfg.n_local_heads, cfg.head_dim, device=device) if kv_cache else None
+            )
+        self.kv_cache_enabled = kv_cache
+        self.freqs_cis = precompute_freqs_cis(max(cfg.block_size, max_seq_length), cfg.head_dim, cfg.rope_base, device=device)
+        self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
+        self.self_mask = torch.eye(max_seq_length, dtype=torch.bool, device=device)
+
+    def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None, left_pad_mask_pos: Optional[Tensor] = None,
+                fully_causal: bool = False) -> Tensor:
+        """idx [B, S] token ids, input_pos [S] positions -> logits [B, S, vocab] (reference :212-248)."""
+        assert self.freqs_cis is not None, "Caches must be initialized first"
+        assert not (fully_causal and left_pad_mask_pos is not None), "Invalid mask"
+        mask = None
+        if not fully_causal:
+            mask = self.causal_mask[None, None, input_pos]
+            if left_pad_mask_pos is not None:
+                visible = torch.arange(mask.size(-1), device=mask.device).view(1, -1) >= left_pad_mask_pos.view(-1, 1)
+                mask = torch.logical_and(mask, visible[:, None, None, :])
+                mask = torch.logical_or(mask, self.self_mask[None, None, input_pos])
+        x = self.tok_embeddings(idx)
+        freqs_cis = self.freqs_cis[input_pos].to(dtype=x.dtype)
+        for layer in self.layers:
+            x = layer(x, input_pos, freqs_cis, mask, fully_causal)
+        return self.output(self.norm(x))
+
+
+class RewardModel(nn.Module):
+    """Backbone whose `output` is a small score head; per-token reward = mean over head rows
+    (reference models/reward_model.py:69-92: `Linear(dim, 2)` head followed by `.mean(-1)`)."""
+
+    def __init__(self, config: ModelArgs, head_rows: int = 2) -> None:
+        super().__init__()
+        self.backbone = Transformer(config)
+        self.backbone.output = nn.Linear(config.dim, head_rows, bias=False)
+
+    def forward(self, idx: Tensor, eos_pos: Optional[Tensor] = None) -> Tensor:
+        input_pos = torch.arange(0, idx.size(-1), device=idx.device)
+        rewards = self.backbone(idx, input_pos=input_pos, fully_causal=True).mean(dim=-1)
+        if eos_pos is not None:
+            rewards = rewards.gather(dim=-1, index=eos_pos.unsqueeze(-1)).squeeze(-1)
+        return rewards
+
+
+def init_random_(model: nn.Module, seed: int = 1234, std: float = 0.02, device=None) -> nn.Module:
+    """Random-init every linear and the embedding with N(0, std), norms with ones, in bfloat16.
+
+    A seeded CPU generator makes the values identical on every machine; `device` only chooses where the
+    parameters end up."""
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    with torch.no_grad():
+        for _, p in model.named_parameters():
+            if p.dim() == 1:
+                new = torch.ones(p.shape, dtype=torch.bfloat16)
+            else:
+                new = (torch.randn(p.shape, generator=gen, dtype=torch.float32) * std).to(torch.bfloat16)
+            p.data = new.to(device if device is not None else p.device)
+    return model

@@ -1,0 +1,292 @@
+"""Tensor-level wrappers of the C ABI (include/e2h_quant.h) and their torch.library registrations.
+
+PyTorch is plumbing here: it owns the device memory (caching allocator) and the stream; every
+arithmetic step runs in the HIP kernels of libe2h_quant.so.  Inputs must live on the GPU -- there is no
+CPU implementation behind these functions.
+
+The `e2h::*` custom ops carry fake (meta) implementations so that modules using them trace under
+torch.compile(fullgraph=True) and capture into HIP graphs (fixed launch geometry, no host sync, no
+allocation outside the caching allocator, kernels on the current stream).
+"""
+
+import ctypes
+
+import torch
+
+from . import _lib
+
+_VALID_GROUPS = (32, 64, 128, 256)
+_VALID_IKT = (2, 4, 8)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _need_gpu(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(
+                "e2h quantized-linear ops run only on the GPU (HIP kernels); got a tensor on %s" % t.device
+            )
+
+
+def _lib_for(t):
+    if t.device.index != torch.cuda.current_device():
+        torch.cuda.set_device(t.device)  # launches go to the current device's stream
+    return _lib.load()
+
+
+# ---------------------------------------------------------------------------------------------
+# int8
+# ---------------------------------------------------------------------------------------------
+
+
+def int8_quantize_per_channel(w):
+    """w [N, K] float32 or bfloat16 on the GPU -> (q int8 [N, K], scales float32 [N]).
+
+    HIP restatement of dynamically_quantize_per_channel(w.float(), -128, 127, torch.int8)
+    (reference models/quantize.py:39-71)."""
+    _need_gpu(w)
+    assert w.dim() == 2
+    if w.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"int8_quantize_per_channel: float32 or bfloat16 expected, got {w.dtype}")
+    w = w.contiguous()
+    n, k = w.shape
+    q = torch.empty((n, k), dtype=torch.int8, device=w.device)
+    scales = torch.empty((n,), dtype=torch.float32, device=w.device)
+    lib = _lib_for(w)
+    rc = lib.e2h_int8_quantize_per_channel(_ptr(w), int(w.dtype == torch.bfloat16), _ptr(q), _ptr(scales), None, n, k, _stream(w))
+    _lib.check(rc, "e2h_int8_quantize_per_channel")
+    return q, scales
+
+
+def _int8_mm_impl(x, q, scales):
+    _need_gpu(x, q, scales)
+    if x.dtype != torch.bfloat16 or q.dtype != torch.int8 or scales.dtype != torch.bfloat16:
+        raise TypeError(f"int8_mm: expected (bfloat16, int8, bfloat16), got ({x.dtype}, {q.dtype}, {scales.dtype})")
+    assert x.dim() == 2 and q.dim() == 2 and scales.dim() == 1
+    m, k = x.shape
+    n = q.shape[0]
+    if q.shape[1] != k or scales.shape[0] != n:
+        raise RuntimeError(f"int8_mm: shape mismatch x{tuple(x.shape)} q{tuple(q.shape)} scales{tuple(scales.shape)}")
+    x, q, scales = x.contiguous(), q.contiguous(), scales.contiguous()
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    if m == 0:
+        return y
+    rc = _lib_for(x).e2h_int8_mm(_ptr(x), _ptr(q), _ptr(scales), _ptr(y), m, n, k, _stream(x))
+    _lib.check(rc, "e2h_int8_mm")
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# int4
+# ---------------------------------------------------------------------------------------------
+
+
+def _check_bf16_2d(w, what):
+    _need_gpu(w)
+    if w.dtype != torch.bfloat16:
+        raise TypeError(f"{what}: bfloat16 weight expected (the reference quantizes int4 in bfloat16), got {w.dtype}")
+    assert w.dim() == 2
+
+
+def int4_group_qparams(w, groupsize):
+    """get_group_qparams (reference models/quantize.py:74-92): bf16 [N, K] -> scales, zeros bf16 [N, K/g]."""
+    _check_bf16_2d(w, "int4_group_qparams")
+    w = w.contiguous()
+    n, k = w.shape
+    scales = torch.empty((n, k // groupsize), dtype=torch.bfloat16, device=w.device)
+    zeros = torch.empty_like(scales)
+    rc = _lib_for(w).e2h_int4_group_qparams(_ptr(w), _ptr(scales), _ptr(zeros), n, k, groupsize, _stream(w))
+    _lib.check(rc, "e2h_int4_group_qparams")
+    return scales, zeros
+
+
+def int4_quantize_from_qparams(w, scales, zeros, groupsize):
+    """group_quantize_tensor_from_qparams (reference :118-144) -> int32 codes [N, K]."""
+    _check_bf16_2d(w, "int4_quantize_from_qparams")
+    _need_gpu(scales, zeros)
+    if scales.dtype != torch.bfloat16 or zeros.dtype != torch.bfloat16:
+        raise TypeError("int4_quantize_from_qparams: bfloat16 qparams expected")
+    w = w.contiguous()
+    n, k = w.shape
+    scales = scales.reshape(n, -1).contiguous()
+    zeros = zeros.reshape(n, -1).contiguous()
+    assert scales.shape == (n, k // groupsize) and zeros.shape == scales.shape
+    codes = torch.empty((n, k), dtype=torch.int32, device=w.device)
+    rc = _lib_for(w).e2h_int4_quantize_from_qparams(_ptr(w), _ptr(scales), _ptr(zeros), _ptr(codes), n, k, groupsize, _stream(w))
+    _lib.check(rc, "e2h_int4_quantize_from_qparams")
+    return codes
+
+
+def int4_group_quantize(w, groupsize):
+    """group_quantize_tensor (reference :147-151) -> (codes int32 [N, K], scales_and_zeros bf16 [K/g, N, 2])."""
+    _check_bf16_2d(w, "int4_group_quantize")
+    w = w.contiguous()
+    n, k = w.shape
+    codes = torch.empty((n, k), dtype=torch.int32, device=w.device)
+    sz = torch.empty((k // groupsize, n, 2), dtype=torch.bfloat16, device=w.device)
+    rc = _lib_for(w).e2h_int4_group_quantize(_ptr(w), _ptr(codes), _ptr(sz), n, k, groupsize, _stream(w))
+    _lib.check(rc, "e2h_int4_group_quantize")
+    return codes, sz
+
+
+def int4_dequantize_codes(codes, scales, zeros, groupsize):
+    """group_dequantize_tensor_from_qparams (reference :154-171) on bfloat16 qparams -> bf16 [N, K]."""
+    _need_gpu(codes, scales, zeros)
+    if codes.dtype != torch.int32 or scales.dtype != torch.bfloat16 or zeros.dtype != torch.bfloat16:
+        raise TypeError("int4_dequantize_codes: expected (int32, bfloat16, bfloat16)")
+    n, k = codes.shape
+    codes = codes.contiguous()
+    scales = scales.reshape(n, -1).contiguous()
+    zeros = zeros.reshape(n, -1).contiguous()
+    assert scales.shape == (n, k // groupsize) and zeros.shape == scales.shape
+    out = torch.empty((n, k), dtype=torch.bfloat16, device=codes.device)
+    rc = _lib_for(codes).e2h_int4_dequantize_codes(_ptr(codes), _ptr(scales), _ptr(zeros), _ptr(out), n, k, groupsize, _stream(codes))
+    _lib.check(rc, "e2h_int4_dequantize_codes")
+    return out
+
+
+def _int4_pack_impl(codes, inner_k_tiles):
+    _need_gpu(codes)
+    if codes.dtype != torch.int32:
+        raise TypeError(f"int4_pack: int32 codes expected, got {codes.dtype}")
+    assert codes.dim() == 2
+    codes = codes.contiguous()
+    n, k = codes.shape
+    if inner_k_tiles not in _VALID_IKT or n % 8 != 0 or k % (16 * inner_k_tiles) != 0:
+        raise RuntimeError(f"int4_pack: need n % 8 == 0, inner_k_tiles in (2,4,8) and k % (16*inner_k_tiles) == 0; got n={n} k={k} ikt={inner_k_tiles}")
+    packed = torch.empty((n // 8, k // (16 * inner_k_tiles), 32, inner_k_tiles // 2), dtype=torch.int32, device=codes.device)
+    rc = _lib_for(codes).e2h_int4_pack(_ptr(codes), _ptr(packed), n, k, inner_k_tiles, _stream(codes))
+    _lib.check(rc, "e2h_int4_pack")
+    return packed
+
+
+def _packed_dims(packed):
+    if packed.dim() != 4 or packed.shape[2] != 32 or packed.dtype != torch.int32:
+        raise RuntimeError(f"expected a tile-packed int32 weight [N/8, K/(16*ikt), 32, ikt/2], got {packed.dtype}{tuple(packed.shape)}")
+    ikt = packed.shape[3] * 2
+    if ikt not in _VALID_IKT:
+        raise RuntimeError(f"tile-packed weight has inner_k_tiles={ikt}, expected 2, 4 or 8")
+    return packed.shape[0] * 8, packed.shape[1] * 16 * ikt, ikt
+
+
+def int4_unpack(packed):
+    """Inverse of int4_pack: tile-packed int32 -> int32 codes [N, K]."""
+    _need_gpu(packed)
+    n, k, ikt = _packed_dims(packed)
+    packed = packed.contiguous()
+    codes = torch.empty((n, k), dtype=torch.int32, device=packed.device)
+    rc = _lib_for(packed).e2h_int4_unpack(_ptr(packed), _ptr(codes), n, k, ikt, _stream(packed))
+    _lib.check(rc, "e2h_int4_unpack")
+    return codes
+
+
+def int4_quantize_pack(w, groupsize, inner_k_tiles):
+    """prepare_int4_weight_and_scales_and_zeros (reference :435-442), fused on the GPU.
+
+    Falls back to the two-kernel route (quantize, then pack) for K not a multiple of 256."""
+    _check_bf16_2d(w, "int4_quantize_pack")
+    w = w.contiguous()
+    n, k = w.shape
+    if groupsize not in _VALID_GROUPS or inner_k_tiles not in _VALID_IKT:
+        raise RuntimeError(f"int4_quantize_pack: unsupported groupsize={groupsize} / inner_k_tiles={inner_k_tiles}")
+    if n % 8 != 0 or k % groupsize != 0 or k % (16 * inner_k_tiles) != 0:
+        raise RuntimeError(f"int4_quantize_pack: unsupported shape n={n} k={k} for groupsize={groupsize}, inner_k_tiles={inner_k_tiles}")
+    if k % 256 != 0:
+        codes, sz = int4_group_quantize(w, groupsize)
+        return _int4_pack_impl(codes, inner_k_tiles), sz
+    packed = torch.empty((n // 8, k // (16 * inner_k_tiles), 32, inner_k_tiles // 2), dtype=torch.int32, device=w.device)
+    sz = torch.empty((k // groupsize, n, 2), dtype=torch.bfloat16, device=w.device)
+    rc = _lib_for(w).e2h_int4_quantize_pack(_ptr(w), _ptr(packed), _ptr(sz), n, k, groupsize, inner_k_tiles, _stream(w))
+    _lib.check(rc, "e2h_int4_quantize_pack")
+    return packed, sz
+
+
+def int4_dequantize(packed, scales_and_zeros, groupsize):
+    """Tile-packed weight + scales_and_zeros -> bf16 [N, K] with the rounding of reference :154-171."""
+    _need_gpu(packed, scales_and_zeros)
+    n, k, ikt = _packed_dims(packed)
+    if scales_and_zeros.dtype != torch.bfloat16 or tuple(scales_and_zeros.shape) != (k // groupsize, n, 2):
+        raise RuntimeError(f"int4_dequantize: scales_and_zeros must be bf16 [{k // groupsize}, {n}, 2], got {scales_and_zeros.dtype}{tuple(scales_and_zeros.shape)}")
+    packed, sz = packed.contiguous(), scales_and_zeros.contiguous()
+    out = torch.empty((n, k), dtype=torch.bfloat16, device=packed.device)
+    rc = _lib_for(packed).e2h_int4_dequantize(_ptr(packed), _ptr(sz), _ptr(out), n, k, groupsize, ikt, _stream(packed))
+    _lib.check(rc, "e2h_int4_dequantize")
+    return out
+
+
+def _int4_mm_impl(x, packed, groupsize, scales_and_zeros):
+    _need_gpu(x, packed, scales_and_zeros)
+    if x.dtype != torch.bfloat16 or scales_and_zeros.dtype != torch.bfloat16:
+        raise TypeError(f"int4_mm: bfloat16 activations and scales_and_zeros expected, got {x.dtype}, {scales_and_zeros.dtype}")
+    assert x.dim() == 2
+    n, k, ikt = _packed_dims(packed)
+    m = x.shape[0]
+    if x.shape[1] != k:
+        raise RuntimeError(f"int4_mm: x has K={x.shape[1]}, packed weight has K={k}")
+    if groupsize not in _VALID_GROUPS or k % groupsize != 0:
+        raise RuntimeError(f"int4_mm: groupsize={groupsize} must be one of {_VALID_GROUPS} and divide K={k}")
+    if tuple(scales_and_zeros.shape) != (k // groupsize, n, 2):
+        raise RuntimeError(f"int4_mm: scales_and_zeros must be [{k // groupsize}, {n}, 2], got {tuple(scales_and_zeros.shape)}")
+    x, packed, sz = x.contiguous(), packed.contiguous(), scales_and_zeros.contiguous()
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    if m == 0:
+        return y
+    rc = _lib_for(x).e2h_int4_mm(_ptr(x), _ptr(packed), _ptr(sz), _ptr(y), m, n, k, groupsize, ikt, _stream(x))
+    _lib.check(rc, "e2h_int4_mm")
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# torch.library registrations (operator boundary that replaces the two aten int4 ops and the
+# F.linear * scales pair of the reference)
+# ---------------------------------------------------------------------------------------------
+
+
+@torch.library.custom_op("e2h::int4_mm", mutates_args=(), device_types="cuda")
+def int4_mm(x: torch.Tensor, packed: torch.Tensor, groupsize: int, scales_and_zeros: torch.Tensor) -> torch.Tensor:
+    """Drop-in for torch.ops.aten._weight_int4pack_mm(x, packed, groupsize, scales_and_zeros)."""
+    return _int4_mm_impl(x, packed, groupsize, scales_and_zeros)
+
+
+@int4_mm.register_fake
+def _(x, packed, groupsize, scales_and_zeros):
+    return x.new_empty((x.shape[0], packed.shape[0] * 8))
+
+
+@torch.library.custom_op("e2h::int4_pack", mutates_args=(), device_types="cuda")
+def int4_pack(codes: torch.Tensor, inner_k_tiles: int) -> torch.Tensor:
+    """Drop-in for torch.ops.aten._convert_weight_to_int4pack(codes_int32[N, K], inner_k_tiles) (PyTorch 2.2 signature)."""
+    return _int4_pack_impl(codes, inner_k_tiles)
+
+
+@int4_pack.register_fake
+def _(codes, inner_k_tiles):
+    n, k = codes.shape
+    return codes.new_empty((n // 8, k // (16 * inner_k_tiles), 32, inner_k_tiles // 2))
+
+
+@torch.library.custom_op("e2h::int8_mm", mutates_args=(), device_types="cuda")
+def int8_mm(x: torch.Tensor, q: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """F.linear(x, q.to(bf16)) * scales  (reference models/quantize.py:428-429) in one kernel."""
+    return _int8_mm_impl(x, q, scales)
+
+
+@int8_mm.register_fake
+def _(x, q, scales):
+    return x.new_empty((x.shape[0], q.shape[0]))
+
+
+def int4_mm_direct(x, packed, groupsize, scales_and_zeros):
+    """Same as the e2h::int4_mm op without the dispatcher round trip (eager hot loops)."""
+    return _int4_mm_impl(x, packed, groupsize, scales_and_zeros)
+
+
+def int8_mm_direct(x, q, scales):
+    return _int8_mm_impl(x, q, scales)

@@ -1,0 +1,126 @@
+/*
+ * e2h_quant.h -- C ABI of libe2h_quant.so: the weight-only quantized linear path of gpt-accelera's
+ * models/quantize.py as hand-written HIP kernels for AMD MI355X (gfx950).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer into memory the caller owns; nothing here allocates, frees
+ *     or synchronises.  Kernels are enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     default stream) and are safe to record into a HIP graph.
+ *   - bfloat16 values travel as uint16_t bit patterns.
+ *   - every entry point returns E2H_OK (0) or a negative E2H_ERR_* code; no exception crosses the ABI.
+ *     e2h_status_string() names a code.
+ *   - "reference" below is gpt-accelera (Edward-Sun/easy-to-hard), file models/quantize.py unless
+ *     another file is named.
+ */
+#ifndef E2H_QUANT_H
+#define E2H_QUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define E2H_ABI_VERSION 1
+
+#define E2H_OK 0
+#define E2H_ERR_NULL_POINTER (-1)      /* a required pointer is NULL */
+#define E2H_ERR_BAD_SHAPE (-2)         /* m/n/k violate the reference's shape asserts */
+#define E2H_ERR_BAD_GROUPSIZE (-3)     /* groupsize not in {32,64,128,256} or does not divide k */
+#define E2H_ERR_BAD_INNER_K_TILES (-4) /* inner_k_tiles not in {2,4,8} or 16*ikt does not divide k */
+#define E2H_ERR_MISALIGNED (-5)        /* a pointer is not aligned as documented */
+#define E2H_ERR_LAUNCH (-6)            /* the HIP runtime rejected the launch */
+#define E2H_ERR_NO_DEVICE (-7)         /* no gfx950 device is current */
+#define E2H_ERR_BAD_OPTION (-8)        /* unknown option name or value out of range */
+
+/* Library identity / diagnostics (no reference counterpart). */
+int e2h_abi_version(void);
+const char *e2h_status_string(int status);
+
+/* Tuning knobs for experiments: name in {"int4_rows_per_wave", "int8_rows_per_wave", "x_transpose"};
+ * value 0 restores the built-in heuristic.  Not thread safe; set before launching. */
+int e2h_set_option(const char *name, int value);
+
+/* ------------------------------------------------------------------------------------------------
+ * int8, per-output-channel symmetric
+ * ---------------------------------------------------------------------------------------------- */
+
+/* dynamically_quantize_per_channel(x, -128, 127, torch.int8), reference :39-71.
+ *   w          [n, k] row-major; float32 if w_is_bf16 == 0 (what the reference's callers pass,
+ *              :357-359 and :388-390), bfloat16 if w_is_bf16 != 0 (converted exactly to float32 on
+ *              the fly, i.e. the same result as quantizing weight.float()).
+ *   q          [n, k] int8 codes.
+ *   scales_f32 [n] float32 scales (the function's second return value); may be NULL.
+ *   scales_bf16[n] the same scales rounded to bfloat16 (what the handler stores, :392); may be NULL.
+ * IEEE float32 division, round-half-even, clamp to [-128, 127]; scale >= float32 eps.
+ * Requires 16-byte aligned w and 4-byte aligned q rows when k % 4 == 0 (any k is accepted). */
+int e2h_int8_quantize_per_channel(const void *w, int w_is_bf16, int8_t *q, float *scales_f32,
+                                  uint16_t *scales_bf16, int64_t n, int64_t k, void *stream);
+
+/* WeightOnlyInt8Linear.forward, reference :428-429:  y = F.linear(x, weight.to(bf16)) * scales.
+ *   x [m, k] bf16, q [n, k] int8, scales [n] bf16, y [m, n] bf16.  float32 accumulation; the result
+ *   is rounded to bfloat16 before and after the multiplication by the scale, as in the reference.
+ * Any m >= 1, n >= 1, k >= 1. */
+int e2h_int8_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int64_t m,
+                int64_t n, int64_t k, void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * int4, group-wise asymmetric
+ * ---------------------------------------------------------------------------------------------- */
+
+/* get_group_qparams(w, 4, groupsize), reference :74-92.  w [n, k] bf16 -> scales, zeros [n, k/g] bf16.
+ * bfloat16 arithmetic: every step is computed in float32 and rounded to bfloat16 (ties to even). */
+int e2h_int4_group_qparams(const uint16_t *w, uint16_t *scales, uint16_t *zeros, int64_t n, int64_t k,
+                           int groupsize, void *stream);
+
+/* group_quantize_tensor_from_qparams(w, scales, zeros, 4, groupsize), reference :118-144.
+ * w [n, k] bf16, scales/zeros [n, k/g] bf16 -> codes [n, k] int32 in 0..15. */
+int e2h_int4_quantize_from_qparams(const uint16_t *w, const uint16_t *scales, const uint16_t *zeros,
+                                   int32_t *codes, int64_t n, int64_t k, int groupsize, void *stream);
+
+/* group_quantize_tensor(w, 4, groupsize), reference :147-151 (get_group_qparams +
+ * group_quantize_tensor_from_qparams + pack_scales_and_zeros :95-109) in one pass.
+ * -> codes [n, k] int32, scales_and_zeros [k/g, n, 2] bf16 ([..,0] scale, [..,1] zero). */
+int e2h_int4_group_quantize(const uint16_t *w, int32_t *codes, uint16_t *scales_and_zeros, int64_t n,
+                            int64_t k, int groupsize, void *stream);
+
+/* torch.ops.aten._convert_weight_to_int4pack(codes, inner_k_tiles) as called at reference :439-441
+ * and :585-587 (PyTorch 2.2.0 CUDA nibble order).
+ * codes [n, k] int32 (0..15) -> packed [n/8, k/(16*ikt), 32, ikt/2] int32.  n % 8 == 0, k % (16*ikt) == 0. */
+int e2h_int4_pack(const int32_t *codes, int32_t *packed, int64_t n, int64_t k, int inner_k_tiles,
+                  void *stream);
+
+/* Inverse of e2h_int4_pack (test aid and checkpoint inspection; no reference counterpart). */
+int e2h_int4_unpack(const int32_t *packed, int32_t *codes, int64_t n, int64_t k, int inner_k_tiles,
+                    void *stream);
+
+/* prepare_int4_weight_and_scales_and_zeros(weight_bf16, groupsize, inner_k_tiles), reference :435-442,
+ * fused: bf16 weight -> tile-packed codes + scales_and_zeros without materialising the int32 codes. */
+int e2h_int4_quantize_pack(const uint16_t *w, int32_t *packed, uint16_t *scales_and_zeros, int64_t n,
+                           int64_t k, int groupsize, int inner_k_tiles, void *stream);
+
+/* group_dequantize_tensor_from_qparams, reference :154-171, applied to the tile-packed weight:
+ * w_out [n, k] bf16 = bf16(bf16((q - 8) * scale) + zero). */
+int e2h_int4_dequantize(const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *w_out,
+                        int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *stream);
+
+/* group_dequantize_tensor_from_qparams(w_int32, scales, zeros, 4, groupsize), reference :154-171, on
+ * plain codes: codes [n, k] int32, scales/zeros [n, k/g] bf16 -> w_out [n, k] bf16
+ * = bf16(bf16((q - 8) * scale) + zero).  Any groupsize >= 2 dividing k. */
+int e2h_int4_dequantize_codes(const int32_t *codes, const uint16_t *scales, const uint16_t *zeros,
+                              uint16_t *w_out, int64_t n, int64_t k, int groupsize, void *stream);
+
+/* torch.ops.aten._weight_int4pack_mm(x, packed, groupsize, scales_and_zeros) as called by
+ * linear_forward_int4, reference :445-453 (WeightOnlyInt4Linear.forward :658-666).
+ *   x [m, k] bf16, packed [n/8, k/(16*ikt), 32, ikt/2] int32, scales_and_zeros [k/g, n, 2] bf16
+ *   -> y [m, n] bf16,  y[m,n] = sum_k x[m,k] * ((q[n,k] - 8) * scale[k/g, n] + zero[k/g, n]),
+ * float32 accumulation.  n % 8 == 0, k % g == 0, k % (16*ikt) == 0, g in {32,64,128,256},
+ * ikt in {2,4,8}; x, packed, scales_and_zeros 16-byte aligned; any m >= 1. */
+int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
+                int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* E2H_QUANT_H */

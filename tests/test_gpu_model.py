@@ -1,0 +1,135 @@
+"""End-to-end GPU checks on a tiny Llama-shaped model: quantize -> save -> load -> run, greedy decoding
+against an oracle model whose linears are the dequantized weights applied with F.linear, and HIP-graph
+replays against eager execution."""
+
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import easy_to_hard_amd as e2h
+from easy_to_hard_amd.generate import GraphedDecodeStep, decode_one_token, generate, model_score, prefill
+from easy_to_hard_amd.model import ModelArgs, RewardModel, Transformer, init_random_
+from oracle import quant_oracle as qo
+from tests.helpers import bf16_to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+class OracleLinear(nn.Module):
+    """x @ W^T in float32 with W = (q - 8) * scale + zero resp. q * scale (dequantize-then-F.linear)."""
+
+    def __init__(self, w_f32):
+        super().__init__()
+        self.register_buffer("w", w_f32)
+
+    def forward(self, x):
+        return torch.nn.functional.linear(x.float(), self.w).to(torch.bfloat16)
+
+
+def _oracle_copy(model_q, mode, g):
+    """Clone of the quantized model with every quantized linear replaced by its float32 oracle."""
+    oracle = copy.deepcopy(model_q)
+    for name, mod in list(oracle.named_modules()):
+        for child_name, child in list(mod.named_children()):
+            if isinstance(child, e2h.WeightOnlyInt4Linear):
+                codes = qo.int4_tile_unpack(child.weight.cpu().numpy(), child.inner_k_tiles)
+                w = qo.int4_dequantize_fp32(codes, bf16_to_np(child.scales_and_zeros), g)
+                setattr(mod, child_name, OracleLinear(torch.from_numpy(w).to(DEV)))
+            elif isinstance(child, e2h.WeightOnlyInt8Linear):
+                w = child.weight.cpu().float() * child.scales.cpu().float()[:, None]
+                setattr(mod, child_name, OracleLinear(w.to(DEV)))
+    return oracle
+
+
+def _tiny(name="tiny-test"):
+    model = Transformer.from_name(name)
+    init_random_(model, seed=1234, std=0.05)
+    return model
+
+
+@pytest.mark.parametrize("name,g", [("tiny-test", 128), ("tiny-gqa-test", 64)])
+def test_int4_checkpoint_roundtrip_and_greedy_decode(tmp_path, name, g):
+    model = _tiny(name)
+    torch.save(model.state_dict(), tmp_path / "model.pth")
+    handler = e2h.WeightOnlyInt4QuantHandler(model, groupsize=g)
+    sd = handler.create_quantized_state_dict()
+    path = tmp_path / f"model_int4.g{g}.pth"
+    torch.save(sd, path)
+    assert sd["layers.0.attention.wqkv.weight"].dtype == torch.int32
+    assert sd["output.scales_and_zeros"].shape == (model.config.dim // g, model.config.vocab_size, 2)
+
+    # runtime path of the reference loader: swap modules on the meta device, load, move to the GPU
+    with torch.device("meta"):
+        rt = Transformer.from_name(name)
+    e2h.WeightOnlyInt4QuantHandler(rt, groupsize=int(path.name.split(".")[-2][1:])).convert_for_runtime()
+    rt.load_state_dict(torch.load(path, mmap=True, weights_only=True), assign=True)
+    rt = rt.to(device=DEV, dtype=torch.bfloat16).eval()
+    assert rt.output.weight.dtype == torch.int32 and rt.output.weight.is_cuda
+
+    oracle = _oracle_copy(rt, "int4", g)
+    bsz, t, new = 4, 12, 10
+    prompt = torch.randint(0, model.config.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(1234)).to(DEV)
+    seq_eager = generate(rt, prompt, new, use_graph=False)
+    seq_graph = generate(rt, prompt, new, use_graph=True)
+    assert torch.equal(seq_eager, seq_graph), "HIP-graph replays must reproduce eager decoding"
+
+    # teacher-forced comparison with the oracle model: same prefix -> logits agree, argmax agrees wherever
+    # the oracle's top-1/top-2 margin exceeds the bf16 noise of the logits
+    oracle.setup_caches(bsz, t + new)
+    rt.setup_caches(bsz, t + new)
+    agree = total = 0
+    for step in range(new):
+        prefix = seq_eager[:, : t + step]
+        pos = torch.arange(0, prefix.shape[1], device=DEV)
+        lq = rt(prefix, pos)[:, -1].float()
+        lo = oracle(prefix, pos)[:, -1].float()
+        err = (lq - lo).abs().max() / lo.abs().max()
+        assert err <= 2e-2, err
+        top2 = lo.topk(2, dim=-1).values
+        margin_ok = (top2[:, 0] - top2[:, 1]) > 4 * (lq - lo).abs().max()
+        agree += int(((lq.argmax(-1) == lo.argmax(-1)) & margin_ok).sum())
+        total += int(margin_ok.sum())
+        assert torch.equal(lq.argmax(-1)[margin_ok], lo.argmax(-1)[margin_ok])
+    assert total > 0 and agree == total
+
+
+def test_int8_on_the_fly_reward_scoring():
+    cfg = ModelArgs.from_name("tiny-test")
+    rm = RewardModel(cfg, head_rows=2)
+    init_random_(rm, seed=7, std=0.05)
+    rm = rm.to(device=DEV, dtype=torch.bfloat16).eval()
+    e2h.WeightOnlyInt8QuantHandler(rm).convert_for_runtime_on_the_fly()
+    assert isinstance(rm.backbone.output, e2h.WeightOnlyInt8Linear) and rm.backbone.output.out_features == 2
+    oracle = _oracle_copy(rm, "int8", None)
+    ids = torch.randint(0, cfg.vocab_size, (3, 40), generator=torch.Generator().manual_seed(1)).to(DEV)
+    r = model_score(rm, ids)
+    r_ref = model_score(oracle, ids)
+    assert r.shape == (3, 40)
+    assert qo.normwise_rel_err(r.float().cpu().numpy(), r_ref.float().cpu().numpy()) <= 2e-2
+
+
+def test_graph_replays_match_eager_every_time():
+    model = _tiny()
+    e2h.WeightOnlyInt4QuantHandler(model, groupsize=32).convert_for_runtime
+    sd = e2h.WeightOnlyInt4QuantHandler(model, groupsize=32).create_quantized_state_dict()
+    e2h.WeightOnlyInt4QuantHandler(model, groupsize=32).convert_for_runtime()
+    model.load_state_dict(sd, assign=True)
+    model = model.to(device=DEV, dtype=torch.bfloat16).eval()
+    bsz = 2
+    model.setup_caches(bsz, 32)
+    prompt = torch.randint(0, 512, (bsz, 8), generator=torch.Generator().manual_seed(3)).to(DEV)
+    cur = prefill(model, prompt, torch.arange(0, 8, device=DEV))
+    stepper = GraphedDecodeStep(model, bsz, DEV)
+    prefill(model, prompt, torch.arange(0, 8, device=DEV))  # restore the cache rows the capture warm-up touched
+    for i in range(6):
+        pos = torch.tensor([8 + i], device=DEV)
+        eager = decode_one_token(model, cur, pos)
+        torch.cuda.synchronize()
+        replay = stepper.step(cur, pos).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(eager, replay), i
+        cur = eager
