@@ -1,0 +1,246 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Workload (default): BASELINE config "random-init Llama-2-7B-architecture model with int4 g128 weight-only
+linears, batch 32, prompt 256, greedy decode, bf16 KV cache".  One step = one decode step of the whole batch
+(161 dequant-GEMV launches + stock attention / norms), replayed from a HIP graph.  `value` is decoded
+tokens per second = batch * steps / time, with everything resident in HBM.
+
+Extra objects on the JSON line:
+  roofline      the dequant-GEMV kernels of one decode step launched back to back (all 161, each on its
+                own weights, 3.5 GB working set per pass so no cache holds it), timed with events on the
+                launch stream: algorithmic bytes / average launch duration against 8 TB/s.
+  cpu_baseline  the reference CPU path (dequantize + F.linear, torch CPU ops) on the host cores for one
+                transformer layer + LM head at the same batch, extrapolated to a full decode step.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--model", default="7B", help="7B (headline) | 34B | tiny-test")
+    ap.add_argument("--mode", default="int4", choices=["int4", "int8"])
+    ap.add_argument("--groupsize", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--prompt", type=int, default=256)
+    ap.add_argument("--max-new", type=int, default=512)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--gemv-reps", type=int, default=20)
+    return ap.parse_args()
+
+
+def quantized_linears(model):
+    import easy_to_hard_amd as e2h
+
+    return [(n, m) for n, m in model.named_modules() if isinstance(m, (e2h.WeightOnlyInt4Linear, e2h.WeightOnlyInt8Linear))]
+
+
+def algorithmic_bytes(mod, m):
+    """HBM bytes one launch has to move: weights + qparams + activations in + out (bf16)."""
+    import easy_to_hard_amd as e2h
+
+    n, k = mod.out_features, mod.in_features
+    if isinstance(mod, e2h.WeightOnlyInt4Linear):
+        return n * k // 2 + (k // mod.groupsize) * n * 4 + m * k * 2 + m * n * 2
+    return n * k + 2 * n + 2 * m * k + 2 * m * n
+
+
+def measure_gemv_roofline(model, batch, reps):
+    """All quantized-linear launches of one decode step, back to back from one HIP graph."""
+    import torch
+
+    dev = torch.device("cuda", 0)
+    lins = quantized_linears(model)
+    xs = {}
+    for _, mod in lins:
+        if mod.in_features not in xs:
+            xs[mod.in_features] = torch.randn((batch, mod.in_features), device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+    def one_pass():
+        out = None
+        for _, mod in lins:
+            out = mod(xs[mod.in_features])
+        return out
+
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        one_pass()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_pass()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    total_s = start.elapsed_time(stop) * 1e-3
+    launches = len(lins) * reps
+    bytes_pass = sum(algorithmic_bytes(mod, batch) for _, mod in lins)
+    avg_launch_s = total_s / launches
+    achieved = bytes_pass * reps / total_s / 1e9
+    return {
+        "bound": "hbm",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "kernel": "int4_skinny_mm_kernel" if "Int4" in type(lins[0][1]).__name__ else "int8_skinny_mm_kernel",
+        "launches_per_step": len(lins),
+        "algorithmic_bytes_per_launch": bytes_pass // len(lins),
+        "avg_launch_us": round(avg_launch_s * 1e6, 3),
+        "gemv_ms_per_step": round(total_s / reps * 1e3, 4),
+    }
+
+
+def measure_cpu_baseline(model, batch, groupsize):
+    """Reference CPU path on the host cores: one layer's five linears + the LM head, extrapolated."""
+    import torch
+
+    import easy_to_hard_amd as e2h
+    from easy_to_hard_amd import ops
+    from oracle import reference_path as rp
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    torch.set_num_threads(cores)
+    backbone = model
+    layer = backbone.layers[0]
+    sample = [layer.attention.wqkv, layer.attention.wo, layer.feed_forward.w1, layer.feed_forward.w3, layer.feed_forward.w2]
+    head = backbone.output
+    gen = torch.Generator().manual_seed(1234)
+
+    def cpu_case(mod):
+        x = torch.randn((batch, mod.in_features), generator=gen).to(torch.bfloat16)
+        if isinstance(mod, e2h.WeightOnlyInt4Linear):
+            codes = ops.int4_unpack(mod.weight).cpu()
+            sz = mod.scales_and_zeros.cpu()
+            return lambda: rp.int4_linear_cpu(x, codes, sz, groupsize)
+        q, s = mod.weight.cpu(), mod.scales.cpu()
+        return lambda: rp.int8_linear_cpu(x, q, s)
+
+    def time_fn(fn, budget_s):
+        fn()
+        times = []
+        t_end = time.perf_counter() + budget_s
+        while len(times) < 2 or (time.perf_counter() < t_end and len(times) < 20):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2]
+
+    layer_s = sum(time_fn(cpu_case(m), 2.5) for m in sample)
+    head_s = time_fn(cpu_case(head), 2.5)
+    n_layer = len(backbone.layers)
+    step_s = layer_s * n_layer + head_s
+    return {
+        "value": round(batch / step_s, 3),
+        "unit": "tok/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"quantized linears of 1 of {n_layer} layers + LM head at batch {batch} (dequantize + F.linear, torch CPU bf16), "
+                  f"median of repeated runs; layer {layer_s * 1e3:.1f} ms, head {head_s * 1e3:.1f} ms; extrapolated to a decode step "
+                  "(linears only, attention excluded)",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from easy_to_hard_amd import _lib
+    from easy_to_hard_amd.generate import GraphedDecodeStep, prefill
+    from easy_to_hard_amd.model import ModelArgs, random_quantized_transformer
+
+    _lib.load()  # no fallback: fail here if the HIP library is not built
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    cfg = ModelArgs.from_name(args.model)
+    t0 = time.time()
+    model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234)
+    torch.cuda.synchronize()
+    build_s = time.time() - t0
+
+    batch, t_prompt = args.batch, args.prompt
+    max_seq = min(t_prompt + args.max_new, cfg.block_size)
+    assert args.warmup + args.steps < max_seq - t_prompt, "warmup + steps must fit in the decode budget"
+    model.setup_caches(batch, max_seq)
+    prompt = torch.randint(0, cfg.vocab_size, (batch, t_prompt), generator=torch.Generator().manual_seed(1234)).to(dev)
+    input_pos = torch.arange(0, t_prompt, device=dev)
+    t0 = time.time()
+    cur = prefill(model, prompt, input_pos)
+    torch.cuda.synchronize()
+    prefill_s = time.time() - t0
+    stepper = GraphedDecodeStep(model, batch, dev)
+    cur = prefill(model, prompt, input_pos)  # the capture warm-up wrote cache row 0
+    pos = torch.tensor([t_prompt], device=dev, dtype=torch.int64)
+    for _ in range(args.warmup):
+        cur = stepper.step(cur, pos).clone()
+        pos += 1
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        cur = stepper.step(cur, pos)
+        pos += 1
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    tok_s = batch * args.steps / elapsed
+
+    roofline = measure_gemv_roofline(model, batch, args.gemv_reps)
+    cpu = None if args.no_cpu_baseline else measure_cpu_baseline(model, batch, args.groupsize)
+
+    line = {
+        "metric": "batched int4 decode tok/s (Llama-7B shape, bs32); dequant-GEMV HBM GB/s % of peak",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"random-init Llama {args.model}-shaped model, {args.mode}"
+                        + (f" g{args.groupsize}" if args.mode == "int4" else "")
+                        + f" weight-only linears, greedy decode, batch {batch}, prompt {t_prompt}, bf16 KV cache of {max_seq} positions, HIP-graph replayed decode step",
+            "batch": batch,
+            "prompt_len": t_prompt,
+            "quantized_linears_per_step": roofline["launches_per_step"],
+            "model_build_s": round(build_s, 2),
+            "prefill_s": round(prefill_s, 3),
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

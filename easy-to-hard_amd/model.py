@@ -271,3 +271,50 @@ def init_random_(model: nn.Module, seed: int = 1234, std: float = 0.02, device=N
                 new = (torch.randn(p.shape, generator=gen, dtype=torch.float32) * std).to(torch.bfloat16)
             p.data = new.to(device if device is not None else p.device)
     return model
+
+
+def random_quantized_transformer(config: ModelArgs, mode: str, groupsize: int = 128, device="cuda", seed: int = 1234,
+                                 std: float = 0.02, reward_head_rows: int = 0) -> nn.Module:
+    """Random-init model of the given shape whose linears are already quantized, built layer by layer on
+    the GPU: each bf16 weight ~ N(0, std) exists only long enough to be quantized by this package's
+    kernels, so a 34B-parameter model never needs its bf16 form in memory.
+
+    mode "int4": WeightOnlyInt4Linear (groupsize, inner_k_tiles 8); mode "int8": WeightOnlyInt8Linear;
+    mode "bf16": plain nn.Linear.  `reward_head_rows` > 0 wraps the backbone in a RewardModel with that many
+    head rows."""
+    import importlib
+
+    qz = importlib.import_module(__package__ + ".quantize")  # the package attribute `quantize` is the function
+
+    dev = torch.device(device)
+    with torch.device("meta"):
+        model = RewardModel(config, reward_head_rows) if reward_head_rows else Transformer(config)
+    backbone = model.backbone if reward_head_rows else model
+    if mode == "int4":
+        qz.WeightOnlyInt4QuantHandler(model, groupsize=groupsize).convert_for_runtime()
+    elif mode == "int8":
+        qz.WeightOnlyInt8QuantHandler(model).convert_for_runtime()
+    else:
+        assert mode == "bf16", mode
+    gen = torch.Generator(device=dev).manual_seed(seed)
+
+    def rand_bf16(shape):
+        return (torch.randn(shape, generator=gen, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+
+    for _, mod in model.named_modules():
+        if isinstance(mod, qz.WeightOnlyInt4Linear):
+            w = rand_bf16((mod.out_features, mod.in_features))
+            mod.weight, mod.scales_and_zeros = qz.prepare_int4_weight_and_scales_and_zeros(w, mod.groupsize, mod.inner_k_tiles)
+        elif isinstance(mod, qz.WeightOnlyInt8Linear):
+            w = rand_bf16((mod.out_features, mod.in_features))
+            q, scales, _ = qz.dynamically_quantize_per_channel(w.float(), -128, 127, torch.int8)
+            mod.weight, mod.scales = q, scales.to(torch.bfloat16)
+        elif isinstance(mod, nn.Linear):
+            mod.weight = nn.Parameter(rand_bf16(tuple(mod.weight.shape)), requires_grad=False)
+        elif isinstance(mod, nn.Embedding):
+            mod.weight = nn.Parameter(rand_bf16(tuple(mod.weight.shape)), requires_grad=False)
+        elif isinstance(mod, RMSNorm):
+            mod.weight = nn.Parameter(torch.ones(mod.weight.shape, dtype=torch.bfloat16, device=dev), requires_grad=False)
+    assert not any(p.is_meta for p in model.parameters()) and not any(b.is_meta for b in model.buffers())
+    backbone.eval()
+    return model.eval()

@@ -73,7 +73,10 @@ def test_int4_mm_exact_small_integers():
     sz = np.zeros((k // g, n, 2), dtype=np.float32)
     sz[..., 0] = 1.0
     sz[..., 1] = 8.0
-    xs = rng.integers(-1, 2, size=(7, k)).astype(np.float32)
+    xs = np.zeros((7, k), dtype=np.float32)
+    for i in range(7):
+        idx = rng.choice(k, size=12, replace=False)       # 12 non-zeros: |y| <= 180 < 256
+        xs[i, idx] = rng.choice([-1.0, 1.0], size=12)
     y = ops.int4_mm_direct(torch.from_numpy(xs).to(torch.bfloat16).to(DEV), torch.from_numpy(qo.int4_tile_pack(codes, ikt)).to(DEV),
                            g, torch.from_numpy(sz).to(torch.bfloat16).to(DEV))
     expect = xs.astype(np.int64) @ codes.T.astype(np.int64)
@@ -168,10 +171,12 @@ def test_int8_mm_config1():
     q, s, q_d, s_d = _int8_case(4096, 4096)
     x = randn_bf16((8, 4096), seed=1235)
     y, err = _check_int8(x, q, s, q_d, s_d)
-    # against the reference's own double rounding the kernel is within one bf16 ulp (accumulation order only)
+    # against the reference's own double rounding only the accumulation order differs: a flip of the first
+    # rounding moves the result by at most one bf16 ulp of the intermediate (2^-7 relative) and the second
+    # rounding can add one more
     y_rr = qo.int8_linear_reference_rounding(bf16_to_np(x), q, s)
     diff = np.abs(bf16_to_np(y) - y_rr)
-    assert np.all(diff <= np.abs(y_rr) * 2.0 ** -7 + 1e-6)
+    assert np.all(diff <= np.abs(y_rr) * 2.0 ** -6 + 1e-6)
     assert np.mean(diff == 0) > 0.95
     print(f"int8 4096x4096 M=8: normwise rel err {err:.3e}, bit-identical to reference rounding: {np.mean(diff == 0):.4f}")
 
@@ -213,7 +218,7 @@ def test_int8_module_and_on_the_fly_handler_with_hooks():
     x = randn_bf16((3, 5, 256), seed=78)
     y = model(x.to(DEV))
     assert calls == ["pre", "post"] and y.shape == (3, 5, 48)
-    q, s, _ = qo.int8_quantize_per_channel(lin.weight.float().cpu().numpy())
+    q, s, _ = qo.int8_quantize_per_channel(lin.weight.detach().float().cpu().numpy())
     np.testing.assert_array_equal(model[0].weight.cpu().numpy(), q)
     np.testing.assert_array_equal(bf16_to_np(model[0].scales), qo.bf16_round(s))
     y_ref = qo.int8_linear_fp32(bf16_to_np(x).reshape(15, 256), q, qo.bf16_round(s)).reshape(3, 5, 48)
