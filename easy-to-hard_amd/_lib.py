@@ -25,7 +25,8 @@ _SIGNATURES = {
     "e2h_int4_quantize_pack": (c_int, [_P, _P, _P, c_int64, c_int64, c_int, c_int, _P]),
     "e2h_int4_dequantize": (c_int, [_P, _P, _P, c_int64, c_int64, c_int, c_int, _P]),
     "e2h_int4_dequantize_codes": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int, _P]),
-    "e2h_int4_mm": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P]),
+    "e2h_int4_mm": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P, c_int64, _P]),
+    "e2h_workspace_bytes": (c_int64, []),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -5,7 +5,7 @@
 
 namespace e2h {
 Options &options() {
-  static Options o = {0, 0, 0};
+  static Options o = {0, 0, 0, 0, 0};
   return o;
 }
 }  // namespace e2h
@@ -33,6 +33,16 @@ extern "C" int e2h_set_option(const char *name, int value) {
   if (!strcmp(name, "int4_rows_per_wave") || !strcmp(name, "int8_rows_per_wave")) {
     if (value != 0 && value != 16 && value != 32 && value != 64) return E2H_ERR_BAD_OPTION;
     (name[3] == '4' ? o.int4_rows_per_wave : o.int8_rows_per_wave) = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int4_k_slices")) {
+    if (value < 0 || value > 16) return E2H_ERR_BAD_OPTION;
+    o.int4_k_slices = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int4_k_groups")) {
+    if (value != 0 && value != 1 && value != 2 && value != 4) return E2H_ERR_BAD_OPTION;
+    o.int4_k_groups = value;
     return E2H_OK;
   }
   if (!strcmp(name, "x_transpose")) {

@@ -35,6 +35,8 @@ __host__ __device__ inline float bf16_round(float f) { return bf16_to_f32(f32_to
 
 struct Options {
   int int4_rows_per_wave;  // 0 = heuristic, else 16/32/64
+  int int4_k_slices;       // 0 = heuristic, else 1..16 workgroups along K
+  int int4_k_groups;       // 0 = heuristic, else 1/2/4 k-groups inside a workgroup
   int int8_rows_per_wave;  // 0 = heuristic, else 16/32/64
   int x_transpose;         // 0 = heuristic
 };

@@ -15,7 +15,7 @@
 //   exactly such a fragment: (word >> 4i) & 0x000F000F is the code pair (k0+8i+2j, k0+8i+2j+1), and
 //   OR-ing 0x43004300 turns it into the bfloat16 pair (128+q, 128+q') with no arithmetic.  A dot product
 //   is invariant under a common permutation of k, so the activation fragment of lane (b, m) is gathered
-//   with the same k order (dwords j, j+4, j+8, j+12 of the 64-byte activation segment) and the weights
+//   with the same k order (dwords b, b+4, b+8, b+12 of each 64-byte activation segment) and the weights
 //   are never re-packed.
 //   The scale and zero are applied to the float32 accumulators once per group:
 //     y[m,n] += s * sum_k x[m,k]*(128+q[n,k]) + (z - 136*s) * sum_k x[m,k]
@@ -23,9 +23,13 @@
 //   accumulator layout).  bf16*bf16 products are exact in float32, so this is more accurate than a
 //   dequantize-to-bf16 kernel.
 //
-// Work decomposition: a workgroup of 4 waves owns 16*T output columns (T tiles of 16 rows of the weight)
-// and 16*MT rows of x; the 4 waves split K (interleaved chunks) and their partial accumulators are
-// summed in a fixed order through LDS, so the result is deterministic.
+// Work decomposition: a workgroup of 4 waves owns 64*T output columns (each wave T tiles of 16 weight rows),
+// 16*MT rows of x and one of S contiguous slices of K.  Per 128-wide k chunk the workgroup stages the
+// activation chunk once into LDS (coalesced 16-byte global loads, scattered so that every MFMA fragment is
+// one conflict-free ds_read_b128), while every wave streams its own packed weights with 128-bit loads kept
+// several chunks ahead in registers.  With S > 1 the slices meet in a workspace: each workgroup stores its
+// float32 partial tile, takes a ticket, and the last one to arrive adds the S partials in slice order -- a
+// fixed order, so results are deterministic -- and writes bf16.
 #include "e2h_common.h"
 
 namespace e2h {
@@ -40,6 +44,7 @@ struct Int4Geom {
   static constexpr int STEPS = CHUNK / 32;               // 32-wide MFMA steps per chunk
   static constexpr int NGRP = CHUNK / G;                 // quantization groups per chunk
   static constexpr int SPG = G / 32;                     // MFMA steps per group
+  static constexpr int PPR = CHUNK / 8;                  // 16-byte activation pieces per row per chunk
 };
 
 template <int N> struct WordVec;
@@ -47,15 +52,27 @@ template <> struct WordVec<1> { typedef uint32_t type; };
 template <> struct WordVec<2> { typedef u32x2_t type; };
 template <> struct WordVec<4> { typedef u32x4_t type; };
 
-constexpr int kWaves = 4;
+constexpr int kWavesN = 4;              // waves that share one activation stream (they split the columns)
+constexpr int kGroupThreads = kWavesN * 64;
+constexpr int kFragBytes = 1024 + 64;   // one MFMA A-fragment block in LDS; the pad skews banks between steps
 
-template <int G, int IKT, int MT, int T>
-struct ChunkRegs {
+template <int G, int IKT, int T>
+struct WeightRegs {
   typedef Int4Geom<G, IKT> Geo;
   uint32_t w[T][Geo::STEPS];
-  u32x4_t xf[MT][Geo::STEPS];
   uint32_t sz[T][Geo::NGRP];
 };
+
+constexpr int kWeightCachePolicy = 2;  // "nt": weights are streamed once, keep them from displacing x and qparams
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also drain every outstanding
+// global load (loads and stores share one counter on this architecture), which would empty the weight
+// prefetch pipeline once per chunk.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ bf16x8_t unpack_word(uint32_t w) {
   constexpr uint32_t kMask = 0x000F000Fu, kMagic = 0x43004300u;  // bf16 128.0 | q  == 128 + q
@@ -67,41 +84,157 @@ __device__ __forceinline__ bf16x8_t unpack_word(uint32_t w) {
   return __builtin_bit_cast(bf16x8_t, u);
 }
 
+// Weight prefetch: a ring of NB register buffers per wave, NB - 1 chunks in flight beyond the one being
+// consumed (about 8 KB per wave: HBM latency here is well over a microsecond, so a CU needs tens of KB in
+// flight).  The main loop is unrolled NB times so that ring slots are compile-time registers.
 template <int G, int IKT, int MT, int T>
-__global__ __launch_bounds__(kWaves * 64, 2) void int4_skinny_mm_kernel(
-    const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
-    uint16_t *__restrict__ y, int M, int N, int K) {
-  typedef Int4Geom<G, IKT> Geo;
-  typedef typename WordVec<Geo::WORDS>::type wvec_t;
+struct Tuning {
+  static constexpr int kChunkWords = T * Int4Geom<G, IKT>::STEPS;  // weight registers per chunk
+  static constexpr int NB = MT >= 4 ? 2 : (kChunkWords <= 4 ? 8 : (kChunkWords <= 8 ? 4 : 2));
+  // Activations are staged into LDS one phase (CPP chunks) at a time, a whole phase ahead of their use, so
+  // the workgroup meets at a barrier once per phase instead of once per chunk.
+  static constexpr int CPP = (MT * Int4Geom<G, IKT>::CHUNK >= 512) ? 2 : 4;
+  // Loads return in issue order, so waiting for an activation load also waits for every weight load issued
+  // before it.  The activation loads of a phase are therefore issued XD phases ahead -- at least as far
+  // ahead (in chunks) as the weight ring -- and by the time they are needed everything older has been
+  // consumed anyway.
+  static constexpr int XD = (NB + CPP - 1) / CPP;
+};
 
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int c = lane & 15;  // column of the MFMA tile (weight row within the 16-row tile) / x row
+// WK = number of k-groups inside the workgroup (each group = kWavesN waves with its own activation stream
+// over a contiguous part of the workgroup's K slice); their accumulators are added through LDS at the end.
+template <int G, int IKT, int MT, int T, int WK>
+__global__ __launch_bounds__(kGroupThreads * WK, (MT >= 4 ? 1 : (WK > 2 ? WK : 2))) void int4_skinny_mm_kernel(
+    const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
+    uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K) {
+  typedef Int4Geom<G, IKT> Geo;
+  typedef WeightRegs<G, IKT, T> wregs_t;
+  constexpr int NB = Tuning<G, IKT, MT, T>::NB;
+  constexpr int PD = NB - 1;
+  constexpr int CPP = Tuning<G, IKT, MT, T>::CPP;
+  constexpr int XD = Tuning<G, IKT, MT, T>::XD;
+  constexpr int U = NB > CPP * XD ? NB : CPP * XD;                  // chunks per unrolled loop body
+  constexpr int kPieces = 16 * MT * Geo::PPR;                       // 16-byte pieces of x per chunk
+  constexpr int kPhasePieces = CPP * kPieces;
+  constexpr int kPiecesPerThread = (kPhasePieces + kGroupThreads - 1) / kGroupThreads;
+  constexpr int kBufBytes = MT * Geo::STEPS * kFragBytes;           // one activation chunk in fragment order
+  constexpr int kStageBytes = CPP * kBufBytes;                      // one phase
+  constexpr int kSlots = T * MT * 4;                                // accumulator registers per lane
+  constexpr int kXBytes = WK * 2 * kStageBytes;
+  constexpr int kRedBytes = (WK - 1) * kWavesN * kSlots * 64 * 4;
+  constexpr int kLdsBytes = kXBytes > kRedBytes ? kXBytes : kRedBytes;
+
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+  __shared__ unsigned s_ticket;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it stays in SGPRs
+  const int wave_n = wave % kWavesN;
+  const int kg = wave / kWavesN;          // k-group of this wave
+  const int tid_g = tid % kGroupThreads;  // thread index within the k-group
+  const int c = lane & 15;  // column of the MFMA tile (weight row within the 16-row tile)
   const int b = lane >> 4;  // k-block of the MFMA
   const int n_tiles8 = N >> 3;
   const int KT = K / Geo::KBLK;
   const int nchunks = K / Geo::CHUNK;
-  const int tile16_0 = blockIdx.x * T;
-  const int m_base = blockIdx.y * (16 * MT);
+  const int S = gridDim.y;
+  const int ks = blockIdx.y;
+  // workgroup slice [C0, C1) of the chunks, then this k-group's part [c0, c1) of it
+  const int C0 = static_cast<int>((static_cast<long long>(nchunks) * ks) / S);
+  const int C1 = static_cast<int>((static_cast<long long>(nchunks) * (ks + 1)) / S);
+  const int c0 = C0 + ((C1 - C0) * kg) / WK;
+  const int c1 = C0 + ((C1 - C0) * (kg + 1)) / WK;
+  const int nloc = c1 - c0;
+  const int nloc_max = (C1 - C0 + WK - 1) / WK;  // trip count, uniform over the workgroup
+  const int tile16_0 = (blockIdx.x * kWavesN + wave_n) * T;
+  const int m_base = blockIdx.z * (16 * MT);
+  uint8_t *const xlds = lds + kg * (2 * kStageBytes);
 
-  const uint32_t *wlane[T];
-  const uint32_t *szlane[T];
+  // ---- addressing: uniform (scalar) base per chunk + constant 32-bit per-lane byte offsets ------------
+  uint32_t wlane[T];   // byte offset of this lane's 16 (or 8 / 4) bytes inside chunk 0 of the packed tensor
+  uint32_t szlane[T];  // byte offset of this lane's column inside one [N] row of (scale, zero) pairs
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     int nt8 = 2 * (tile16_0 + t) + (c >> 3);
     nt8 = nt8 < n_tiles8 ? nt8 : n_tiles8 - 1;
-    wlane[t] = wp + (static_cast<size_t>(nt8) * KT * 32 + ((c & 7) * 4 + b)) * Geo::WORDS;
+    wlane[t] = static_cast<uint32_t>((static_cast<size_t>(nt8) * KT * 32 + ((c & 7) * 4 + b)) * Geo::WORDS * 4);
     int ncol = 16 * (tile16_0 + t) + c;
     ncol = ncol < N ? ncol : N - 1;
-    szlane[t] = sz + ncol;
+    szlane[t] = static_cast<uint32_t>(ncol) * 4u;
   }
-  const uint16_t *xlane[MT];
+  // Buffer addressing: resource (scalar) + scalar byte offset of the chunk + the lane's constant offset,
+  // so a load costs no vector ALU work at all.  Every tensor is smaller than 4 GB (checked on the host).
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(wp, static_cast<uint32_t>(static_cast<size_t>(N) * K / 2));
+  const __amdgpu_buffer_rsrc_t sz_rsrc = make_rsrc(sz, static_cast<uint32_t>(static_cast<size_t>(K / G) * N * 4));
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
+
+  auto load_weights = [&](wregs_t &r, int ci) {
+    const uint32_t wchunk = static_cast<uint32_t>(ci) * (Geo::NBLK * 32 * Geo::WORDS * 4);
+    const uint32_t szchunk = static_cast<uint32_t>(ci) * Geo::NGRP * N * 4;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int row = m_base + 16 * mt + c;
+    for (int t = 0; t < T; ++t) {
+#pragma unroll
+      for (int blk = 0; blk < Geo::NBLK; ++blk) {
+        const uint32_t so = wchunk + blk * (32 * Geo::WORDS * 4);
+        if constexpr (Geo::WORDS == 4) {
+          const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[t], so, kWeightCachePolicy);
+#pragma unroll
+          for (int p = 0; p < 4; ++p) r.w[t][blk * 4 + p] = v[p];
+        } else if constexpr (Geo::WORDS == 2) {
+          const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, wlane[t], so, kWeightCachePolicy);
+          r.w[t][blk * 2] = v[0];
+          r.w[t][blk * 2 + 1] = v[1];
+        } else {
+          r.w[t][blk] = __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, wlane[t], so, kWeightCachePolicy);
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < Geo::NGRP; ++g)
+        r.sz[t][g] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, szlane[t], szchunk + g * N * 4, 0);
+    }
+  };
+
+  // ---- cooperative activation staging (per k-group) ------------------------------------------------
+  // piece p of a phase: chunk q = p / kPieces of the phase; within the chunk row = p' / PPR and 16-byte piece
+  // `within` = p' % PPR of that row's CHUNK-wide segment; step s = within / 4, u = within % 4.  Its dword j
+  // belongs to lane (b = j, m = row % 16), register u.
+  uint32_t xsrc[kPiecesPerThread];  // byte offset of the piece inside chunk 0 of x
+  int xdst[kPiecesPerThread];
+  int xq[kPiecesPerThread];
+#pragma unroll
+  for (int i = 0; i < kPiecesPerThread; ++i) {
+    const int p = tid_g + i * kGroupThreads;
+    const int q = (p / kPieces) < CPP ? (p / kPieces) : CPP - 1;
+    const int pc = p % kPieces;
+    int row = pc / Geo::PPR;
+    const int within = pc % Geo::PPR;
+    const int s = within >> 2, u = within & 3;
+    xq[i] = q;
+    xdst[i] = q * kBufBytes + ((row >> 4) * Geo::STEPS + s) * kFragBytes + (row & 15) * 16 + u * 4;
+    row += m_base;
     row = row < M ? row : M - 1;
-    xlane[mt] = x + static_cast<size_t>(row) * K + 2 * b;
+    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + within * 8) * 2);
   }
+  auto chunk_at = [&](int i) {
+    const int ci = c0 + (i < nloc ? i : nloc - 1);
+    return ci < C0 ? C0 : ci;  // a group without chunks re-reads the first chunk of the slice
+  };
+  auto load_x = [&](u32x4_t (&r)[kPiecesPerThread], int phase) {
+#pragma unroll
+    for (int i = 0; i < kPiecesPerThread; ++i)
+      if (kPhasePieces % kGroupThreads == 0 || tid_g + i * kGroupThreads < kPhasePieces)
+        r[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(chunk_at(phase * CPP + xq[i])) * (Geo::CHUNK * 2), 0);
+  };
+  auto store_x = [&](const u32x4_t (&r)[kPiecesPerThread], int parity) {
+    uint8_t *buf = xlds + (parity & 1) * kStageBytes;
+#pragma unroll
+    for (int i = 0; i < kPiecesPerThread; ++i)
+      if (kPhasePieces % kGroupThreads == 0 || tid_g + i * kGroupThreads < kPhasePieces) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint32_t *>(buf + xdst[i] + j * 256) = r[i][j];
+      }
+  };
 
   f32x4_t acc[T][MT];
 #pragma unroll
@@ -109,38 +242,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void int4_skinny_mm_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  auto load_chunk = [&](ChunkRegs<G, IKT, MT, T> &r, int ci) {
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-#pragma unroll
-      for (int blk = 0; blk < Geo::NBLK; ++blk) {
-        const size_t kb = static_cast<size_t>(ci) * Geo::NBLK + blk;
-        wvec_t v = *reinterpret_cast<const wvec_t *>(wlane[t] + kb * (32 * Geo::WORDS));
-        if constexpr (Geo::WORDS == 1) {
-          r.w[t][blk] = v;
-        } else {
-#pragma unroll
-          for (int p = 0; p < Geo::WORDS; ++p) r.w[t][blk * Geo::WORDS + p] = v[p];
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < Geo::NGRP; ++g)
-        r.sz[t][g] = szlane[t][(static_cast<size_t>(ci) * Geo::NGRP + g) * N];
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const uint16_t *xp = xlane[mt] + static_cast<size_t>(ci) * Geo::CHUNK;
-#pragma unroll
-      for (int s = 0; s < Geo::STEPS; ++s) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) r.xf[mt][s][i] = *reinterpret_cast<const uint32_t *>(xp + 32 * s + 8 * i);
-      }
-    }
-  };
-
   const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
 
-  auto compute_chunk = [&](const ChunkRegs<G, IKT, MT, T> &r) {
+  auto compute_chunk = [&](const wregs_t &r, int parity, int q, uint32_t live) {
+    const uint8_t *buf = xlds + (parity & 1) * kStageBytes + q * kBufBytes + lane * 16;
+    bf16x8_t xf[MT][Geo::STEPS];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int s = 0; s < Geo::STEPS; ++s)
+        xf[mt][s] = *reinterpret_cast<const bf16x8_t *>(buf + (mt * Geo::STEPS + s) * kFragBytes);
     // group sums of x, already in accumulator layout (every column holds the same sum)
     f32x4_t xs[MT][Geo::NGRP];
 #pragma unroll
@@ -150,7 +261,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void int4_skinny_mm_kernel(
         f32x4_t s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < Geo::SPG; ++s)
-          s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, r.xf[mt][g * Geo::SPG + s]), ones, s4, 0, 0, 0);
+          s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][g * Geo::SPG + s], ones, s4, 0, 0, 0);
         xs[mt][g] = s4;
       }
     }
@@ -166,9 +277,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void int4_skinny_mm_kernel(
           const bf16x8_t wf = unpack_word(r.w[t][g * Geo::SPG + s]);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
-            part[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, r.xf[mt][g * Geo::SPG + s]), wf, part[mt], 0, 0, 0);
+            part[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][g * Geo::SPG + s], wf, part[mt], 0, 0, 0);
         }
-        const uint32_t szw = r.sz[t][g];
+        const uint32_t szw = r.sz[t][g] & live;  // live == 0 turns the chunk into a no-op (scale = zero = 0)
         const float scale = __builtin_bit_cast(float, szw << 16);
         const float zero = __builtin_bit_cast(float, szw & 0xFFFF0000u);
         const float zc = __builtin_fmaf(-136.0f, scale, zero);
@@ -186,91 +297,206 @@ __global__ __launch_bounds__(kWaves * 64, 2) void int4_skinny_mm_kernel(
     }
   };
 
-  ChunkRegs<G, IKT, MT, T> bufA, bufB;
-  int ci = wave;
-  if (ci < nchunks) load_chunk(bufA, ci);
-  while (ci < nchunks) {
-    const int c1 = ci + kWaves;
-    if (c1 < nchunks) load_chunk(bufB, c1);
-    compute_chunk(bufA);
-    if (c1 >= nchunks) break;
-    const int c2 = c1 + kWaves;
-    if (c2 < nchunks) load_chunk(bufA, c2);
-    compute_chunk(bufB);
-    ci = c2;
+  // ---- main pipeline -----------------------------------------------------------------------------
+  // The loop body is branch-free so that the compiler can count outstanding loads exactly and never waits
+  // for younger prefetches: chunk indices past the end of the group's part are clamped to a valid chunk (the
+  // loads hit cache, the arithmetic is neutralised with live = 0), and the trip count is rounded up to U.
+  wregs_t ring[NB];
+  u32x4_t xstage[XD][kPiecesPerThread];
+  if (C1 > C0) {
+#pragma unroll
+    for (int d = 0; d < XD; ++d) load_x(xstage[d], d);
+#pragma unroll
+    for (int i = 0; i < PD; ++i) load_weights(ring[i], chunk_at(i));
+    store_x(xstage[0], 0);
+    lds_barrier();
+    // invariant at the top of phase ph: LDS stage (ph & 1) holds the activations of phase ph, register set
+    // (ph + d) % XD holds (or is still receiving) phase ph + d for d = 1 .. XD-1, set ph % XD is free
+    for (int base = 0; base < nloc_max; base += U) {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const int i = base + j;
+        const int phase = i / CPP;
+        const uint32_t live = i < nloc ? 0xFFFFFFFFu : 0u;
+#ifndef E2H_DBG_NO_X
+        if (j % CPP == 0) load_x(xstage[(j / CPP) % XD], phase + XD);
+#endif
+        load_weights(ring[(j + PD) % NB], chunk_at(i + PD));
+#ifdef E2H_DBG_NO_COMPUTE
+        {
+          uint32_t h = 0;
+#pragma unroll
+          for (int t = 0; t < T; ++t) {
+#pragma unroll
+            for (int s2 = 0; s2 < Geo::STEPS; ++s2) h ^= ring[j % NB].w[t][s2];
+#pragma unroll
+            for (int g2 = 0; g2 < Geo::NGRP; ++g2) h ^= ring[j % NB].sz[t][g2];
+          }
+          acc[0][0][0] += __builtin_bit_cast(float, h & live & 0x3FFFFFFFu);
+        }
+#else
+        compute_chunk(ring[j % NB], phase, j % CPP, live);
+#endif
+#ifndef E2H_DBG_NO_X
+        if (j % CPP == CPP - 1) {
+          store_x(xstage[(j / CPP + 1) % XD], phase + 1);
+          lds_barrier();
+        }
+#endif
+      }
+    }
   }
 
-  // cross-wave reduction in a fixed order, then bf16 store
-  __shared__ float red[kWaves][T * MT * 4][64];
+  // ---- epilogue 1: add the k-groups of this workgroup through LDS (fixed order) --------------------
+  if constexpr (WK > 1) {
+    float *red = reinterpret_cast<float *>(lds);
+    if (kg > 0) {
+      float *mine = red + (static_cast<size_t>(kg - 1) * kWavesN + wave_n) * kSlots * 64 + lane;
 #pragma unroll
-  for (int t = 0; t < T; ++t)
+      for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) mine[((t * MT + mt) * 4 + q) * 64] = acc[t][mt][q];
+    }
+    lds_barrier();
+    if (kg == 0) {
+#pragma unroll
+      for (int g2 = 1; g2 < WK; ++g2) {
+        const float *other = red + (static_cast<size_t>(g2 - 1) * kWavesN + wave_n) * kSlots * 64 + lane;
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[t][mt][q] += other[((t * MT + mt) * 4 + q) * 64];
+      }
+    }
+  }
+
+  // ---- epilogue 2: combine the K slices of different workgroups ------------------------------------
+  // Partial tiles and the ticket travel as device-scope relaxed atomics (written through to, and read from,
+  // the memory side, so no cache write-back or invalidate is needed); the stores are complete before the
+  // ticket is taken, and the loads are issued after it has been observed.
+  if (S > 1) {
+    const size_t tile_floats = static_cast<size_t>(kWavesN) * kSlots * 64;
+    const size_t wg_tile = static_cast<size_t>(blockIdx.z) * gridDim.x + blockIdx.x;
+    if (kg == 0) {
+      float *mine = ws_partial + (wg_tile * S + ks) * tile_floats + static_cast<size_t>(wave_n) * kSlots * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            __hip_atomic_store(mine + ((t * MT + mt) * 4 + q) * 64, acc[t][mt][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(ws_ticket + wg_tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != static_cast<unsigned>(S - 1)) return;
+    if (tid == 0) __hip_atomic_store(ws_ticket + wg_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    if (kg == 0) {
+      const float *all = ws_partial + wg_tile * S * tile_floats + static_cast<size_t>(wave_n) * kSlots * 64 + lane;
+      // slice order 0, 1, .., S-1 for every element, whichever workgroup arrived last
+      for (int s2 = 0; s2 < S; ++s2) {
+        float v[kSlots];
+#pragma unroll
+        for (int slot = 0; slot < kSlots; ++slot)
+          v[slot] = __hip_atomic_load(all + s2 * tile_floats + slot * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int slot = (t * MT + mt) * 4 + q;
+              acc[t][mt][q] = s2 == 0 ? v[slot] : acc[t][mt][q] + v[slot];
+            }
+      }
+    }
+  }
+  if (kg != 0) return;
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const int n = 16 * (tile16_0 + t) + c;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) red[wave][(t * MT + mt) * 4 + q][lane] = acc[t][mt][q];
-  __syncthreads();
-#pragma unroll
-  for (int it = 0; it < T * MT; ++it) {
-    const int e = it * (kWaves * 64) + threadIdx.x;
-    const int L = e & 63;
-    const int slot = e >> 6;
-    const int q = slot & 3;
-    const int mt = (slot >> 2) % MT;
-    const int t = (slot >> 2) / MT;
-    float s = red[0][slot][L];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) s += red[w][slot][L];
-    const int n = 16 * (tile16_0 + t) + (L & 15);
-    const int m = m_base + 16 * mt + 4 * (L >> 4) + q;
-    if (n < N && m < M) y[static_cast<size_t>(m) * N + n] = f32_to_bf16_rne(s);
+      for (int q = 0; q < 4; ++q) {
+        const int m = m_base + 16 * mt + 4 * b + q;
+        if (n < N && m < M) y[static_cast<size_t>(m) * N + n] = f32_to_bf16_rne(acc[t][mt][q]);
+      }
   }
 }
 
-template <int G, int IKT, int MT, int T>
-int launch(const uint16_t *x, const int32_t *packed, const uint16_t *sz, uint16_t *y, int M, int N, int K,
-           hipStream_t stream) {
-  const int tiles16 = (N + 15) / 16;
-  dim3 grid((tiles16 + T - 1) / T, (M + 16 * MT - 1) / (16 * MT));
-  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T>), grid, dim3(kWaves * 64), 0, stream, x,
-                     reinterpret_cast<const uint32_t *>(packed), reinterpret_cast<const uint32_t *>(sz), y, M, N, K);
+struct LaunchArgs {
+  const uint16_t *x;
+  const int32_t *packed;
+  const uint16_t *sz;
+  uint16_t *y;
+  float *ws_partial;
+  unsigned *ws_ticket;
+  int M, N, K, S;
+  hipStream_t stream;
+};
+
+template <int G, int IKT, int MT, int T, int WK>
+int launch(const LaunchArgs &a) {
+  const int tiles16 = (a.N + 15) / 16;
+  dim3 grid((tiles16 + kWavesN * T - 1) / (kWavesN * T), a.S, (a.M + 16 * MT - 1) / (16 * MT));
+  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WK>), grid, dim3(kGroupThreads * WK), 0, a.stream, a.x,
+                     reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz), a.y,
+                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K);
   return launch_status();
 }
 
 template <int G, int IKT>
-int dispatch_mt_t(int mt, int t, const uint16_t *x, const int32_t *packed, const uint16_t *sz, uint16_t *y,
-                  int M, int N, int K, hipStream_t stream) {
+int dispatch_mt_t(int mt, int t, int wk, const LaunchArgs &a) {
   if constexpr (IKT == 8 && G <= 128) {
-#define E2H_CASE(MTV, TV) \
-  if (mt == MTV && t == TV) return launch<G, IKT, MTV, TV>(x, packed, sz, y, M, N, K, stream);
-    E2H_CASE(1, 1) E2H_CASE(1, 2) E2H_CASE(1, 4)
-    E2H_CASE(2, 1) E2H_CASE(2, 2) E2H_CASE(2, 4)
-    E2H_CASE(4, 1) E2H_CASE(4, 2)
+#define E2H_CASE(MTV, TV, WKV) \
+  if (mt == MTV && t == TV && wk == WKV) return launch<G, IKT, MTV, TV, WKV>(a);
+    E2H_CASE(1, 1, 1) E2H_CASE(1, 2, 1) E2H_CASE(1, 4, 1)
+    E2H_CASE(2, 1, 1) E2H_CASE(2, 2, 1) E2H_CASE(2, 4, 1)
+    E2H_CASE(1, 1, 2) E2H_CASE(1, 2, 2) E2H_CASE(1, 4, 2)
+    E2H_CASE(2, 1, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 4, 2)
+    E2H_CASE(1, 1, 4) E2H_CASE(1, 2, 4)
+    E2H_CASE(4, 1, 1) E2H_CASE(4, 2, 1)
 #undef E2H_CASE
-    return launch<G, IKT, 4, 2>(x, packed, sz, y, M, N, K, stream);
+    return launch<G, IKT, 4, 2, 1>(a);
   } else {
-    // rarely used geometries: one column tile per workgroup keeps the register footprint small
-    if (mt == 1) return launch<G, IKT, 1, 1>(x, packed, sz, y, M, N, K, stream);
-    if (mt == 2) return launch<G, IKT, 2, 1>(x, packed, sz, y, M, N, K, stream);
-    return launch<G, IKT, 4, 1>(x, packed, sz, y, M, N, K, stream);
+    // rarely used geometries: one column tile per wave keeps the register footprint small
+    if (mt == 1) return launch<G, IKT, 1, 1, 1>(a);
+    if constexpr (G == 256) {
+      return launch<G, IKT, 2, 1, 1>(a);  // 256-wide chunks: four row tiles of x would not fit the LDS budget
+    } else {
+      if (mt == 2) return launch<G, IKT, 2, 1, 1>(a);
+      return launch<G, IKT, 4, 1, 1>(a);
+    }
   }
 }
 
 template <int G>
-int dispatch_ikt(int ikt, int mt, int t, const uint16_t *x, const int32_t *packed, const uint16_t *sz,
-                 uint16_t *y, int M, int N, int K, hipStream_t stream) {
+int dispatch_ikt(int ikt, int mt, int t, int wk, const LaunchArgs &a) {
   switch (ikt) {
-    case 2: return dispatch_mt_t<G, 2>(mt, t, x, packed, sz, y, M, N, K, stream);
-    case 4: return dispatch_mt_t<G, 4>(mt, t, x, packed, sz, y, M, N, K, stream);
-    default: return dispatch_mt_t<G, 8>(mt, t, x, packed, sz, y, M, N, K, stream);
+    case 2: return dispatch_mt_t<G, 2>(mt, t, wk, a);
+    case 4: return dispatch_mt_t<G, 4>(mt, t, wk, a);
+    default: return dispatch_mt_t<G, 8>(mt, t, wk, a);
   }
 }
+
+constexpr size_t kTicketBytes = 64 * 1024;  // 16384 tickets
+constexpr int kCUs = 256;
 
 }  // namespace
 }  // namespace e2h
 
+extern "C" int64_t e2h_workspace_bytes(void) { return static_cast<int64_t>(e2h::kTicketBytes) + (int64_t{32} << 20); }
+
 extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
                            uint16_t *y, int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles,
-                           void *stream) {
+                           void *workspace, int64_t workspace_bytes, void *stream) {
   using namespace e2h;
   if (!x || !packed || !scales_and_zeros || !y) return E2H_ERR_NULL_POINTER;
   if (groupsize != 32 && groupsize != 64 && groupsize != 128 && groupsize != 256) return E2H_ERR_BAD_GROUPSIZE;
@@ -280,23 +506,80 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   if (k % (16 * inner_k_tiles) != 0) return E2H_ERR_BAD_INNER_K_TILES;
   if (!aligned16(x) || !aligned16(packed) || !aligned16(scales_and_zeros) || (reinterpret_cast<uintptr_t>(y) & 1u))
     return E2H_ERR_MISALIGNED;
-  const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
-  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  // columns per workgroup: enough workgroups to cover the chip a few times over, otherwise as many
-  // weight tiles per activation fragment as possible
+  if (workspace && !aligned16(workspace)) return E2H_ERR_MISALIGNED;
+  if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
+  LaunchArgs a;
+  a.x = x; a.packed = packed; a.sz = scales_and_zeros; a.y = y;
+  a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
+  a.stream = static_cast<hipStream_t>(stream);
+  int mt = a.M <= 16 ? 1 : (a.M <= 32 ? 2 : 4);
+  if (groupsize == 256 && mt == 4) mt = 2;
+  const int m_chunks = (a.M + 16 * mt - 1) / (16 * mt);
+  const int tiles16 = (a.N + 15) / 16;
+  const int chunk = groupsize > 16 * inner_k_tiles ? groupsize : 16 * inner_k_tiles;
+  const int nchunks = a.K / chunk;
+  const bool wide_ok = inner_k_tiles == 8 && groupsize <= 128;
+
+  // Tile width T (weight tiles per wave) and K slices S: aim for >= 2 workgroups per CU; prefer wide
+  // tiles (activation fragments are reused T times) and few slices (partials cost S tile round trips).
   int t = options().int4_rows_per_wave / 16;
+  int s = options().int4_k_slices;
+  const bool have_ws = workspace && workspace_bytes >= static_cast<int64_t>(kTicketBytes) + (int64_t{1} << 20);
   if (t != 1 && t != 2 && t != 4) {
-    const int tiles16 = (N + 15) / 16;
     t = 1;
-    if (tiles16 >= 2 * 1024) t = 2;
-    if (tiles16 >= 4 * 1024 && mt <= 2) t = 4;
+    if (wide_ok) {
+      const int target = 2 * kCUs;
+      for (int cand = (mt == 4 ? 2 : 4); cand >= 1; cand >>= 1) {
+        const int blocks = (tiles16 + kWavesN * cand - 1) / (kWavesN * cand) * m_chunks;
+        const int max_s = have_ws ? (cand >= 4 ? 2 : 4) : 1;
+        if (blocks * max_s >= target || cand == 1) { t = cand; break; }
+      }
+    }
   }
+  if (!wide_ok) t = 1;
   if (mt == 4 && t == 4) t = 2;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (groupsize) {
-    case 32: return dispatch_ikt<32>(inner_k_tiles, mt, t, x, packed, scales_and_zeros, y, M, N, K, s);
-    case 64: return dispatch_ikt<64>(inner_k_tiles, mt, t, x, packed, scales_and_zeros, y, M, N, K, s);
-    case 128: return dispatch_ikt<128>(inner_k_tiles, mt, t, x, packed, scales_and_zeros, y, M, N, K, s);
-    default: return dispatch_ikt<256>(inner_k_tiles, mt, t, x, packed, scales_and_zeros, y, M, N, K, s);
+  int wk = options().int4_k_groups;
+  if (wk != 1 && wk != 2 && wk != 4) wk = 1;
+  if (!wide_ok || mt == 4) wk = 1;
+  if (wk == 4 && (t == 4 || mt == 2)) wk = 2;
+  const int n_blocks = (tiles16 + kWavesN * t - 1) / (kWavesN * t);
+  if (s < 1) {
+    s = 1;
+    if (have_ws) {
+      const int blocks = n_blocks * m_chunks;
+      while (s < 8 && blocks * s < kCUs && nchunks / (2 * s) >= 4) s *= 2;
+    }
   }
+  if (s > nchunks) s = nchunks;
+  if (s > 1) {
+    // workspace layout: [tickets | float partial tiles]
+    const int64_t tile_floats = static_cast<int64_t>(kWavesN) * t * mt * 4 * 64;
+    const int64_t need = static_cast<int64_t>(kTicketBytes) + static_cast<int64_t>(n_blocks) * m_chunks * s * tile_floats * 4;
+    if (!have_ws || need > workspace_bytes || static_cast<int64_t>(n_blocks) * m_chunks * 4 > static_cast<int64_t>(kTicketBytes)) s = 1;
+  }
+  a.S = s;
+  a.ws_ticket = reinterpret_cast<unsigned *>(workspace);
+  a.ws_partial = workspace ? reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + kTicketBytes) : nullptr;
+  // The kernels address x through a 32-bit buffer descriptor: slice M so that every launch sees < 4 GB
+  // of activations (and a grid within limits).  Decode-sized calls take a single pass.
+  const int64_t rows_by_bytes = ((int64_t{1} << 32) - 1) / (2 * static_cast<int64_t>(a.K));
+  const int64_t rows_by_grid = int64_t{65535} * 16 * mt;
+  int64_t max_rows = rows_by_bytes < rows_by_grid ? rows_by_bytes : rows_by_grid;
+  max_rows -= max_rows % (16 * mt);
+  if (max_rows < 16 * mt) return E2H_ERR_BAD_SHAPE;
+  const int m_total = a.M;
+  for (int64_t m0 = 0; m0 < m_total; m0 += max_rows) {
+    a.x = x + m0 * a.K;
+    a.y = y + m0 * a.N;
+    a.M = static_cast<int>(m_total - m0 < max_rows ? m_total - m0 : max_rows);
+    int rc;
+    switch (groupsize) {
+      case 32: rc = dispatch_ikt<32>(inner_k_tiles, mt, t, wk, a); break;
+      case 64: rc = dispatch_ikt<64>(inner_k_tiles, mt, t, wk, a); break;
+      case 128: rc = dispatch_ikt<128>(inner_k_tiles, mt, t, wk, a); break;
+      default: rc = dispatch_ikt<256>(inner_k_tiles, mt, t, wk, a); break;
+    }
+    if (rc != E2H_OK) return rc;
+  }
+  return E2H_OK;
 }

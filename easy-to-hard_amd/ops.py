@@ -35,6 +35,19 @@ def _need_gpu(*tensors):
             )
 
 
+_workspaces = {}
+
+
+def _workspace(device):
+    """One zero-initialised scratch tensor per device for the split-K tickets and partial tiles.  All launches
+    that use it are issued on the current stream, which orders them."""
+    ws = _workspaces.get(device.index)
+    if ws is None:
+        ws = torch.zeros(int(_lib.load().e2h_workspace_bytes()), dtype=torch.uint8, device=device)
+        _workspaces[device.index] = ws
+    return ws
+
+
 def _lib_for(t):
     if t.device.index != torch.cuda.current_device():
         torch.cuda.set_device(t.device)  # launches go to the current device's stream
@@ -238,7 +251,8 @@ def _int4_mm_impl(x, packed, groupsize, scales_and_zeros):
     y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     if m == 0:
         return y
-    rc = _lib_for(x).e2h_int4_mm(_ptr(x), _ptr(packed), _ptr(sz), _ptr(y), m, n, k, groupsize, ikt, _stream(x))
+    ws = _workspace(x.device)
+    rc = _lib_for(x).e2h_int4_mm(_ptr(x), _ptr(packed), _ptr(sz), _ptr(y), m, n, k, groupsize, ikt, _ptr(ws), ws.numel(), _stream(x))
     _lib.check(rc, "e2h_int4_mm")
     return y
 

@@ -38,7 +38,7 @@ extern "C" {
 int e2h_abi_version(void);
 const char *e2h_status_string(int status);
 
-/* Tuning knobs for experiments: name in {"int4_rows_per_wave", "int8_rows_per_wave", "x_transpose"};
+/* Tuning knobs for experiments: name in {"int4_rows_per_wave", "int4_k_slices", "int8_rows_per_wave", "x_transpose"};
  * value 0 restores the built-in heuristic.  Not thread safe; set before launching. */
 int e2h_set_option(const char *name, int value);
 
@@ -116,9 +116,17 @@ int e2h_int4_dequantize_codes(const int32_t *codes, const uint16_t *scales, cons
  *   x [m, k] bf16, packed [n/8, k/(16*ikt), 32, ikt/2] int32, scales_and_zeros [k/g, n, 2] bf16
  *   -> y [m, n] bf16,  y[m,n] = sum_k x[m,k] * ((q[n,k] - 8) * scale[k/g, n] + zero[k/g, n]),
  * float32 accumulation.  n % 8 == 0, k % g == 0, k % (16*ikt) == 0, g in {32,64,128,256},
- * ikt in {2,4,8}; x, packed, scales_and_zeros 16-byte aligned; any m >= 1. */
+ * ikt in {2,4,8}; x, packed, scales_and_zeros 16-byte aligned; any m >= 1.
+ *   workspace  optional scratch of workspace_bytes bytes (16-byte aligned; e2h_workspace_bytes() is the
+ *              recommended size) that lets small problems split K across workgroups.  It must be zero
+ *              when first used and is left zeroed where it matters by every launch; launches that share
+ *              it must be ordered on one stream.  NULL / 0 selects the single-slice kernels. */
 int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
-                int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *stream);
+                int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *workspace,
+                int64_t workspace_bytes, void *stream);
+
+/* Recommended size in bytes of the workspace accepted by the matmul entry points (no reference counterpart). */
+int64_t e2h_workspace_bytes(void);
 
 #ifdef __cplusplus
 }
