@@ -5,7 +5,7 @@
 
 namespace e2h {
 Options &options() {
-  static Options o = {0, 0, 0, 0, 0};
+  static Options o = {0, 0, 0, 0, 0, 0};
   return o;
 }
 }  // namespace e2h
@@ -43,6 +43,11 @@ extern "C" int e2h_set_option(const char *name, int value) {
   if (!strcmp(name, "int4_k_groups")) {
     if (value != 0 && value != 1 && value != 2 && value != 4) return E2H_ERR_BAD_OPTION;
     o.int4_k_groups = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int4_col_waves")) {
+    if (value < 0 || value > 4) return E2H_ERR_BAD_OPTION;
+    o.int4_col_waves = value;
     return E2H_OK;
   }
   if (!strcmp(name, "x_transpose")) {

@@ -37,6 +37,7 @@ struct Options {
   int int4_rows_per_wave;  // 0 = heuristic, else 16/32/64
   int int4_k_slices;       // 0 = heuristic, else 1..16 workgroups along K
   int int4_k_groups;       // 0 = heuristic, else 1/2/4 k-groups inside a workgroup
+  int int4_col_waves;      // 0 = heuristic, else 1..4 column waves per k-group
   int int8_rows_per_wave;  // 0 = heuristic, else 16/32/64
   int x_transpose;         // 0 = heuristic
 };

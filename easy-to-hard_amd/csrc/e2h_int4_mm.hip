@@ -52,8 +52,6 @@ template <> struct WordVec<1> { typedef uint32_t type; };
 template <> struct WordVec<2> { typedef u32x2_t type; };
 template <> struct WordVec<4> { typedef u32x4_t type; };
 
-constexpr int kWavesN = 4;              // waves that share one activation stream (they split the columns)
-constexpr int kGroupThreads = kWavesN * 64;
 constexpr int kFragBytes = 1024 + 64;   // one MFMA A-fragment block in LDS; the pad skews banks between steps
 
 template <int G, int IKT, int T>
@@ -74,26 +72,41 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, ui
 // prefetch pipeline once per chunk.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-__device__ __forceinline__ bf16x8_t unpack_word(uint32_t w) {
-  constexpr uint32_t kMask = 0x000F000Fu, kMagic = 0x43004300u;  // bf16 128.0 | q  == 128 + q
+// (w >> 4i) & 0x000F000F | 0x43004300: two codes -> the bfloat16 pair (128 + q, 128 + q').  The mask lives
+// in an SGPR and the magic in a VGPR so that each pair is one v_and_or_b32 (this ISA's VOP3 encoding takes no
+// literal and only one scalar operand); the asm statements only keep the compiler from folding them back
+// into literals.
+struct UnpackConsts {
+  uint32_t mask, magic;
+};
+__device__ __forceinline__ UnpackConsts unpack_consts() {
+  UnpackConsts c;
+  asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(c.mask));
+  asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(c.magic));
+  return c;
+}
+__device__ __forceinline__ bf16x8_t unpack_word(uint32_t w, const UnpackConsts &c) {
   u32x4_t u;
-  u[0] = (w & kMask) | kMagic;
-  u[1] = ((w >> 4) & kMask) | kMagic;
-  u[2] = ((w >> 8) & kMask) | kMagic;
-  u[3] = ((w >> 12) & kMask) | kMagic;
+  u[0] = (w & c.mask) | c.magic;
+  u[1] = ((w >> 4) & c.mask) | c.magic;
+  u[2] = ((w >> 8) & c.mask) | c.magic;
+  u[3] = ((w >> 12) & c.mask) | c.magic;
   return __builtin_bit_cast(bf16x8_t, u);
 }
 
 // Weight prefetch: a ring of NB register buffers per wave, NB - 1 chunks in flight beyond the one being
 // consumed (about 8 KB per wave: HBM latency here is well over a microsecond, so a CU needs tens of KB in
 // flight).  The main loop is unrolled NB times so that ring slots are compile-time registers.
-template <int G, int IKT, int MT, int T>
+template <int G, int IKT, int MT, int T, int WN, int WK>
 struct Tuning {
   static constexpr int kChunkWords = T * Int4Geom<G, IKT>::STEPS;  // weight registers per chunk
-  static constexpr int NB = MT >= 4 ? 2 : (kChunkWords <= 4 ? 8 : (kChunkWords <= 8 ? 4 : 2));
+  // few waves per workgroup: deep ring; many waves: the other waves of the SIMD cover the latency
+  static constexpr int NB = MT >= 4 ? 2 : (kChunkWords <= 4 ? (WN * WK <= 4 ? 8 : 4) : (kChunkWords <= 8 ? 4 : 2));
   // Activations are staged into LDS one phase (CPP chunks) at a time, a whole phase ahead of their use, so
   // the workgroup meets at a barrier once per phase instead of once per chunk.
-  static constexpr int CPP = (MT * Int4Geom<G, IKT>::CHUNK >= 512) ? 2 : 4;
+  static constexpr int kChunkLds = MT * Int4Geom<G, IKT>::STEPS * kFragBytes;  // one chunk of x in LDS
+  static constexpr int kLdsBudget = (WK >= 4 ? 144 : 72) * 1024;               // both stages of all k-groups
+  static constexpr int CPP = (WK * 2 * 4 * kChunkLds <= kLdsBudget) ? 4 : ((WK * 2 * 2 * kChunkLds <= kLdsBudget) ? 2 : 1);
   // Loads return in issue order, so waiting for an activation load also waits for every weight load issued
   // before it.  The activation loads of a phase are therefore issued XD phases ahead -- at least as far
   // ahead (in chunks) as the weight ring -- and by the time they are needed everything older has been
@@ -101,18 +114,21 @@ struct Tuning {
   static constexpr int XD = (NB + CPP - 1) / CPP;
 };
 
-// WK = number of k-groups inside the workgroup (each group = kWavesN waves with its own activation stream
-// over a contiguous part of the workgroup's K slice); their accumulators are added through LDS at the end.
-template <int G, int IKT, int MT, int T, int WK>
-__global__ __launch_bounds__(kGroupThreads * WK, (MT >= 4 ? 1 : (WK > 2 ? WK : 2))) void int4_skinny_mm_kernel(
+// WN = waves that share one activation stream and split the workgroup's columns; WK = number of k-groups
+// inside the workgroup (each group = WN waves with its own activation stream over a contiguous part of the
+// workgroup's K slice); the k-groups' accumulators are added through LDS at the end.
+template <int G, int IKT, int MT, int T, int WN, int WK>
+__global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
     uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K) {
   typedef Int4Geom<G, IKT> Geo;
   typedef WeightRegs<G, IKT, T> wregs_t;
-  constexpr int NB = Tuning<G, IKT, MT, T>::NB;
+  constexpr int kWavesN = WN;
+  constexpr int kGroupThreads = WN * 64;
+  constexpr int NB = Tuning<G, IKT, MT, T, WN, WK>::NB;
   constexpr int PD = NB - 1;
-  constexpr int CPP = Tuning<G, IKT, MT, T>::CPP;
-  constexpr int XD = Tuning<G, IKT, MT, T>::XD;
+  constexpr int CPP = Tuning<G, IKT, MT, T, WN, WK>::CPP;
+  constexpr int XD = Tuning<G, IKT, MT, T, WN, WK>::XD;
   constexpr int U = NB > CPP * XD ? NB : CPP * XD;                  // chunks per unrolled loop body
   constexpr int kPieces = 16 * MT * Geo::PPR;                       // 16-byte pieces of x per chunk
   constexpr int kPhasePieces = CPP * kPieces;
@@ -242,6 +258,7 @@ __global__ __launch_bounds__(kGroupThreads * WK, (MT >= 4 ? 1 : (WK > 2 ? WK : 2
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+  const UnpackConsts uc = unpack_consts();
   const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
 
   auto compute_chunk = [&](const wregs_t &r, int parity, int q, uint32_t live) {
@@ -274,7 +291,7 @@ __global__ __launch_bounds__(kGroupThreads * WK, (MT >= 4 ? 1 : (WK > 2 ? WK : 2
         for (int mt = 0; mt < MT; ++mt) part[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < Geo::SPG; ++s) {
-          const bf16x8_t wf = unpack_word(r.w[t][g * Geo::SPG + s]);
+          const bf16x8_t wf = unpack_word(r.w[t][g * Geo::SPG + s], uc);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             part[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][g * Geo::SPG + s], wf, part[mt], 0, 0, 0);
@@ -442,47 +459,54 @@ struct LaunchArgs {
   hipStream_t stream;
 };
 
-template <int G, int IKT, int MT, int T, int WK>
+template <int G, int IKT, int MT, int T, int WN, int WK>
 int launch(const LaunchArgs &a) {
   const int tiles16 = (a.N + 15) / 16;
-  dim3 grid((tiles16 + kWavesN * T - 1) / (kWavesN * T), a.S, (a.M + 16 * MT - 1) / (16 * MT));
-  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WK>), grid, dim3(kGroupThreads * WK), 0, a.stream, a.x,
+  dim3 grid((tiles16 + WN * T - 1) / (WN * T), a.S, (a.M + 16 * MT - 1) / (16 * MT));
+  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
                      reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz), a.y,
                      a.ws_partial, a.ws_ticket, a.M, a.N, a.K);
   return launch_status();
 }
 
+// (T, WN, WK) shapes instantiated for the common geometry (inner_k_tiles 8, group size <= 128)
+struct Shape {
+  int t, wn, wk;
+};
+constexpr Shape kShapes[] = {{1, 4, 1}, {1, 4, 2}, {1, 4, 4}, {1, 3, 4}, {1, 2, 4}, {1, 2, 2}, {1, 1, 4},
+                             {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {2, 3, 2}, {4, 4, 1}};
+
 template <int G, int IKT>
-int dispatch_mt_t(int mt, int t, int wk, const LaunchArgs &a) {
+int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
   if constexpr (IKT == 8 && G <= 128) {
-#define E2H_CASE(MTV, TV, WKV) \
-  if (mt == MTV && t == TV && wk == WKV) return launch<G, IKT, MTV, TV, WKV>(a);
-    E2H_CASE(1, 1, 1) E2H_CASE(1, 2, 1) E2H_CASE(1, 4, 1)
-    E2H_CASE(2, 1, 1) E2H_CASE(2, 2, 1) E2H_CASE(2, 4, 1)
-    E2H_CASE(1, 1, 2) E2H_CASE(1, 2, 2) E2H_CASE(1, 4, 2)
-    E2H_CASE(2, 1, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 4, 2)
-    E2H_CASE(1, 1, 4) E2H_CASE(1, 2, 4)
-    E2H_CASE(4, 1, 1) E2H_CASE(4, 2, 1)
+#define E2H_CASE(TV, WNV, WKV)                                                  \
+  if (sh.t == TV && sh.wn == WNV && sh.wk == WKV) {                             \
+    if (mt == 1) return launch<G, IKT, 1, TV, WNV, WKV>(a);                     \
+    if (mt == 2) return launch<G, IKT, 2, TV, WNV, WKV>(a);                     \
+  }
+    E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 4, 4) E2H_CASE(1, 3, 4) E2H_CASE(1, 2, 4) E2H_CASE(1, 2, 2)
+    E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1)
 #undef E2H_CASE
-    return launch<G, IKT, 4, 2, 1>(a);
+    if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1>(a);
+    return launch<G, IKT, 4, 1, 4, 1>(a);
   } else {
     // rarely used geometries: one column tile per wave keeps the register footprint small
-    if (mt == 1) return launch<G, IKT, 1, 1, 1>(a);
+    if (mt == 1) return launch<G, IKT, 1, 1, 4, 1>(a);
     if constexpr (G == 256) {
-      return launch<G, IKT, 2, 1, 1>(a);  // 256-wide chunks: four row tiles of x would not fit the LDS budget
+      return launch<G, IKT, 2, 1, 4, 1>(a);  // 256-wide chunks: four row tiles of x would not fit the LDS budget
     } else {
-      if (mt == 2) return launch<G, IKT, 2, 1, 1>(a);
-      return launch<G, IKT, 4, 1, 1>(a);
+      if (mt == 2) return launch<G, IKT, 2, 1, 4, 1>(a);
+      return launch<G, IKT, 4, 1, 4, 1>(a);
     }
   }
 }
 
 template <int G>
-int dispatch_ikt(int ikt, int mt, int t, int wk, const LaunchArgs &a) {
+int dispatch_ikt(int ikt, int mt, Shape sh, const LaunchArgs &a) {
   switch (ikt) {
-    case 2: return dispatch_mt_t<G, 2>(mt, t, wk, a);
-    case 4: return dispatch_mt_t<G, 4>(mt, t, wk, a);
-    default: return dispatch_mt_t<G, 8>(mt, t, wk, a);
+    case 2: return dispatch_shape<G, 2>(mt, sh, a);
+    case 4: return dispatch_shape<G, 4>(mt, sh, a);
+    default: return dispatch_shape<G, 8>(mt, sh, a);
   }
 }
 
@@ -520,40 +544,34 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   const int nchunks = a.K / chunk;
   const bool wide_ok = inner_k_tiles == 8 && groupsize <= 128;
 
-  // Tile width T (weight tiles per wave) and K slices S: aim for >= 2 workgroups per CU; prefer wide
-  // tiles (activation fragments are reused T times) and few slices (partials cost S tile round trips).
-  int t = options().int4_rows_per_wave / 16;
-  int s = options().int4_k_slices;
+  // Decomposition: a workgroup = WN column waves x WK k-groups, each wave T tiles of 16 weight rows; S
+  // workgroups share a column block along K.
   const bool have_ws = workspace && workspace_bytes >= static_cast<int64_t>(kTicketBytes) + (int64_t{1} << 20);
-  if (t != 1 && t != 2 && t != 4) {
-    t = 1;
-    if (wide_ok) {
-      const int target = 2 * kCUs;
-      for (int cand = (mt == 4 ? 2 : 4); cand >= 1; cand >>= 1) {
-        const int blocks = (tiles16 + kWavesN * cand - 1) / (kWavesN * cand) * m_chunks;
-        const int max_s = have_ws ? (cand >= 4 ? 2 : 4) : 1;
-        if (blocks * max_s >= target || cand == 1) { t = cand; break; }
-      }
-    }
+  // Measured on MI355X: 8 waves per workgroup (4 column waves x 2 k-groups, one tile each) is the best
+  // all-round shape -- two waves per SIMD overlap arithmetic with memory waits -- and narrow matrices
+  // additionally split K over S workgroups until about 3/4 of the CUs have one.
+  Shape sh = {1, 4, 1};
+  int s = 1;
+  if (wide_ok && mt <= 2) {
+    sh = Shape{1, 4, 2};
+    const int blocks = ((tiles16 + 3) / 4) * m_chunks;
+    if (have_ws)
+      while (s < 4 && blocks * s < (3 * kCUs) / 4 && nchunks / (2 * s * sh.wk) >= 4) s *= 2;
+  } else if (wide_ok) {
+    sh = Shape{tiles16 >= 2 * kCUs * 4 ? 2 : 1, 4, 1};
   }
-  if (!wide_ok) t = 1;
-  if (mt == 4 && t == 4) t = 2;
-  int wk = options().int4_k_groups;
-  if (wk != 1 && wk != 2 && wk != 4) wk = 1;
-  if (!wide_ok || mt == 4) wk = 1;
-  if (wk == 4 && (t == 4 || mt == 2)) wk = 2;
-  const int n_blocks = (tiles16 + kWavesN * t - 1) / (kWavesN * t);
-  if (s < 1) {
-    s = 1;
-    if (have_ws) {
-      const int blocks = n_blocks * m_chunks;
-      while (s < 8 && blocks * s < kCUs && nchunks / (2 * s) >= 4) s *= 2;
-    }
+  const int opt_t = options().int4_rows_per_wave / 16, opt_wk = options().int4_k_groups, opt_wn = options().int4_col_waves;
+  if (wide_ok && mt <= 2 && (opt_t || opt_wk || opt_wn)) {
+    Shape want = {opt_t ? opt_t : sh.t, opt_wn ? opt_wn : sh.wn, opt_wk ? opt_wk : sh.wk};
+    for (const Shape &cand : kShapes)
+      if (cand.t == want.t && cand.wn == want.wn && cand.wk == want.wk) sh = cand;
   }
+  if (options().int4_k_slices > 0) s = options().int4_k_slices;
   if (s > nchunks) s = nchunks;
+  const int n_blocks = (tiles16 + sh.wn * sh.t - 1) / (sh.wn * sh.t);
   if (s > 1) {
     // workspace layout: [tickets | float partial tiles]
-    const int64_t tile_floats = static_cast<int64_t>(kWavesN) * t * mt * 4 * 64;
+    const int64_t tile_floats = static_cast<int64_t>(sh.wn) * sh.t * mt * 4 * 64;
     const int64_t need = static_cast<int64_t>(kTicketBytes) + static_cast<int64_t>(n_blocks) * m_chunks * s * tile_floats * 4;
     if (!have_ws || need > workspace_bytes || static_cast<int64_t>(n_blocks) * m_chunks * 4 > static_cast<int64_t>(kTicketBytes)) s = 1;
   }
@@ -574,10 +592,10 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     a.M = static_cast<int>(m_total - m0 < max_rows ? m_total - m0 : max_rows);
     int rc;
     switch (groupsize) {
-      case 32: rc = dispatch_ikt<32>(inner_k_tiles, mt, t, wk, a); break;
-      case 64: rc = dispatch_ikt<64>(inner_k_tiles, mt, t, wk, a); break;
-      case 128: rc = dispatch_ikt<128>(inner_k_tiles, mt, t, wk, a); break;
-      default: rc = dispatch_ikt<256>(inner_k_tiles, mt, t, wk, a); break;
+      case 32: rc = dispatch_ikt<32>(inner_k_tiles, mt, sh, a); break;
+      case 64: rc = dispatch_ikt<64>(inner_k_tiles, mt, sh, a); break;
+      case 128: rc = dispatch_ikt<128>(inner_k_tiles, mt, sh, a); break;
+      default: rc = dispatch_ikt<256>(inner_k_tiles, mt, sh, a); break;
     }
     if (rc != E2H_OK) return rc;
   }
