@@ -26,6 +26,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per dequant-GEMV launch (fetched + written) from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --gemv-only`, scaled by a 256 MiB copy; the summary with the commands is in
+# profiles/int4_skinny_mm_7b_decode_bs32.md.  Counters cannot be read from inside this process, so the figure is
+# recorded here for the configuration it was measured on and reported as null for any other.
+MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32): 29_440_000}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -40,6 +46,8 @@ def parse_args():
     ap.add_argument("--max-new", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--gemv-reps", type=int, default=20)
+    ap.add_argument("--gemv-only", action="store_true",
+                    help="only the back-to-back dequant-GEMV pass plus a 256 MiB calibration copy (for counter runs)")
     return ap.parse_args()
 
 
@@ -59,7 +67,7 @@ def algorithmic_bytes(mod, m):
     return n * k + 2 * n + 2 * m * k + 2 * m * n
 
 
-def measure_gemv_roofline(model, batch, reps):
+def measure_gemv_roofline(model, batch, reps, traffic_key=None):
     """All quantized-linear launches of one decode step, back to back from one HIP graph."""
     import torch
 
@@ -104,7 +112,7 @@ def measure_gemv_roofline(model, batch, reps):
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(traffic_key),
         "kernel": "int4_skinny_mm_kernel" if "Int4" in type(lins[0][1]).__name__ else "int8_skinny_mm_kernel",
         "launches_per_step": len(lins),
         "algorithmic_bytes_per_launch": bytes_pass // len(lins),
@@ -186,6 +194,17 @@ def main():
     build_s = time.time() - t0
 
     batch, t_prompt = args.batch, args.prompt
+    if args.gemv_only:
+        # counter-collection mode: the GEMV pass and a plain copy of known size (its FETCH_SIZE / WRITE_SIZE
+        # readings calibrate the counters: 256 MiB read, 256 MiB written per copy)
+        roofline = measure_gemv_roofline(model, batch, args.gemv_reps, (args.model, args.mode, args.groupsize, batch))
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"roofline": roofline, "calibration_copy_bytes": src.numel()}))
+        return
     max_seq = min(t_prompt + args.max_new, cfg.block_size)
     assert args.warmup + args.steps < max_seq - t_prompt, "warmup + steps must fit in the decode budget"
     model.setup_caches(batch, max_seq)
@@ -210,7 +229,7 @@ def main():
     elapsed = time.perf_counter() - t0
     tok_s = batch * args.steps / elapsed
 
-    roofline = measure_gemv_roofline(model, batch, args.gemv_reps)
+    roofline = measure_gemv_roofline(model, batch, args.gemv_reps, (args.model, args.mode, args.groupsize, batch))
     cpu = None if args.no_cpu_baseline else measure_cpu_baseline(model, batch, args.groupsize)
 
     line = {
