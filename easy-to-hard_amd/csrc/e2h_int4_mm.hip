@@ -487,6 +487,7 @@ int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
     E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 4, 4) E2H_CASE(1, 3, 4) E2H_CASE(1, 2, 4) E2H_CASE(1, 2, 2)
     E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1)
 #undef E2H_CASE
+    if (sh.t == 4) return launch<G, IKT, 4, 4, 4, 1>(a);
     if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1>(a);
     return launch<G, IKT, 4, 1, 4, 1>(a);
   } else {
@@ -558,7 +559,12 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     if (have_ws)
       while (s < 4 && blocks * s < (3 * kCUs) / 4 && nchunks / (2 * s * sh.wk) >= 4) s *= 2;
   } else if (wide_ok) {
-    sh = Shape{tiles16 >= 2 * kCUs * 4 ? 2 : 1, 4, 1};
+    // many rows of x (prefill, scoring): every weight fragment feeds four row tiles straight from registers;
+    // wide column blocks keep the LDS traffic for activation fragments below the MFMA rate
+    const int opt_t4 = options().int4_rows_per_wave / 16;
+    const long long wgs4 = static_cast<long long>((tiles16 + 15) / 16) * m_chunks;
+    (void)wgs4;
+    sh = Shape{opt_t4 ? opt_t4 : (static_cast<long long>((tiles16 + 7) / 8) * m_chunks >= kCUs ? 2 : 1), 4, 1};  // T = 2 measured best (830 TFLOP/s at M = 8192)
   }
   const int opt_t = options().int4_rows_per_wave / 16, opt_wk = options().int4_k_groups, opt_wn = options().int4_col_waves;
   if (wide_ok && mt <= 2 && (opt_t || opt_wk || opt_wn)) {
