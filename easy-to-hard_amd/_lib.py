@@ -16,7 +16,7 @@ _SIGNATURES = {
     "e2h_status_string": (c_char_p, [c_int]),
     "e2h_set_option": (c_int, [c_char_p, c_int]),
     "e2h_int8_quantize_per_channel": (c_int, [_P, c_int, _P, _P, _P, c_int64, c_int64, _P]),
-    "e2h_int8_mm": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, _P]),
+    "e2h_int8_mm": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, _P, c_int64, _P]),
     "e2h_int4_group_qparams": (c_int, [_P, _P, _P, c_int64, c_int64, c_int, _P]),
     "e2h_int4_quantize_from_qparams": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int, _P]),
     "e2h_int4_group_quantize": (c_int, [_P, _P, _P, c_int64, c_int64, c_int, _P]),

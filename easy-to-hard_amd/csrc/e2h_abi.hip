@@ -5,7 +5,7 @@
 
 namespace e2h {
 Options &options() {
-  static Options o = {0, 0, 0, 0, 0, 0};
+  static Options o = {};
   return o;
 }
 }  // namespace e2h
@@ -48,6 +48,20 @@ extern "C" int e2h_set_option(const char *name, int value) {
   if (!strcmp(name, "int4_col_waves")) {
     if (value < 0 || value > 4) return E2H_ERR_BAD_OPTION;
     o.int4_col_waves = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int8_k_groups")) {
+    if (value < 0 || value > 2) return E2H_ERR_BAD_OPTION;
+    o.int8_k_groups = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int8_force_generic")) {
+    o.int8_force_generic = value != 0;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int8_k_slices")) {
+    if (value < 0 || value > 16) return E2H_ERR_BAD_OPTION;
+    o.int8_k_slices = value;
     return E2H_OK;
   }
   if (!strcmp(name, "x_transpose")) {

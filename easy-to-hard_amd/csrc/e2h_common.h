@@ -39,9 +39,28 @@ struct Options {
   int int4_k_groups;       // 0 = heuristic, else 1/2/4 k-groups inside a workgroup
   int int4_col_waves;      // 0 = heuristic, else 1..4 column waves per k-group
   int int8_rows_per_wave;  // 0 = heuristic, else 16/32/64
+  int int8_k_groups;       // 0 = heuristic, else 1/2
+  int int8_k_slices;       // 0 = heuristic, else 1..16
+  int int8_force_generic;  // 1 = always use the generic (bounds-checked) int8 kernel
   int x_transpose;         // 0 = heuristic
 };
 Options &options();
+
+#if defined(__HIPCC__)
+// Buffer resource for raw buffer loads: base pointer + byte size (< 4 GB), no swizzle.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also drain every outstanding
+// global load (loads and stores share one counter on this architecture), which would empty a register
+// prefetch pipeline once per use.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+#endif
+
+// streaming int8 matmul (e2h_int8_stream.hip)
+int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int M, int N, int K, void *workspace,
+                   int64_t workspace_bytes, hipStream_t stream);
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -63,14 +63,6 @@ struct WeightRegs {
 
 constexpr int kWeightCachePolicy = 2;  // "nt": weights are streamed once, keep them from displacing x and qparams
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
-}
-
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also drain every outstanding
-// global load (loads and stores share one counter on this architecture), which would empty the weight
-// prefetch pipeline once per chunk.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // (w >> 4i) & 0x000F000F | 0x43004300: two codes -> the bfloat16 pair (128 + q, 128 + q').  The mask lives
 // in an SGPR and the magic in a VGPR so that each pair is one v_and_or_b32 (this ISA's VOP3 encoding takes no

@@ -44,7 +44,7 @@ struct ChunkRegs8 {
 // GUARD: element-wise bounds-checked loads (any K, any alignment).  Otherwise K % 64 == 0 and 16-byte
 // aligned rows are required.
 template <int MT, int T, bool GUARD>
-__global__ __launch_bounds__(kWaves * 64, 2) void int8_skinny_mm_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
+__global__ __launch_bounds__(kWaves * 64, 2) void int8_generic_mm_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
                                                                         const uint16_t *__restrict__ scales, uint16_t *__restrict__ y,
                                                                         int M, int N, int K) {
   const int lane = threadIdx.x & 63;
@@ -182,9 +182,9 @@ int launch(bool guard, const uint16_t *x, const int8_t *q, const uint16_t *scale
            hipStream_t stream) {
   dim3 grid((N + 16 * T - 1) / (16 * T), (M + 16 * MT - 1) / (16 * MT));
   if (guard)
-    hipLaunchKernelGGL((int8_skinny_mm_kernel<MT, T, true>), grid, dim3(kWaves * 64), 0, stream, x, q, scales, y, M, N, K);
+    hipLaunchKernelGGL((int8_generic_mm_kernel<MT, T, true>), grid, dim3(kWaves * 64), 0, stream, x, q, scales, y, M, N, K);
   else
-    hipLaunchKernelGGL((int8_skinny_mm_kernel<MT, T, false>), grid, dim3(kWaves * 64), 0, stream, x, q, scales, y, M, N, K);
+    hipLaunchKernelGGL((int8_generic_mm_kernel<MT, T, false>), grid, dim3(kWaves * 64), 0, stream, x, q, scales, y, M, N, K);
   return launch_status();
 }
 
@@ -192,13 +192,17 @@ int launch(bool guard, const uint16_t *x, const int8_t *q, const uint16_t *scale
 }  // namespace e2h
 
 extern "C" int e2h_int8_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int64_t m, int64_t n,
-                           int64_t k, void *stream) {
+                           int64_t k, void *workspace, int64_t workspace_bytes, void *stream) {
   using namespace e2h;
   if (!x || !q || !scales || !y) return E2H_ERR_NULL_POINTER;
   if (m < 1 || n < 1 || k < 1 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if ((reinterpret_cast<uintptr_t>(x) & 1u) || (reinterpret_cast<uintptr_t>(y) & 1u) || (reinterpret_cast<uintptr_t>(scales) & 1u))
     return E2H_ERR_MISALIGNED;
   const int M = static_cast<int>(m), N = static_cast<int>(n), K = static_cast<int>(k);
+  if (workspace && !aligned16(workspace)) return E2H_ERR_MISALIGNED;
+  // streaming kernel: K in whole 128-wide chunks, 16-byte aligned rows, weight matrix below 4 GB
+  if ((K % 128) == 0 && aligned16(x) && aligned16(q) && n * k < (int64_t{1} << 32) && !options().int8_force_generic)
+    return int8_stream_mm(x, q, scales, y, M, N, K, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
   const bool guard = (K % kChunk) != 0 || !aligned16(x) || !aligned16(q);
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   int t = options().int8_rows_per_wave / 16;

@@ -1,0 +1,363 @@
+// int8 per-channel dequant GEMV / skinny GEMM / GEMM, streaming version (K % 128 == 0, 16-byte aligned rows).
+//
+// Replaces  F.linear(x, weight.to(bf16)) * scales  (reference models/quantize.py:428-429).
+//
+//   q int8 [N][K] row-major (checkpoint layout), scales bf16 [N], x bf16 [M][K], y bf16 [M][N].
+//
+// Same pipeline as the int4 kernel: a workgroup = WN column waves x WK k-groups, each wave T tiles of 16 weight
+// rows and 16*MT rows of x; S workgroups may split K.  Lane L = 16*b + c of v_mfma_f32_16x16x32_bf16 owns weight row
+// n0 + c; per 64-wide half chunk it loads the 16 consecutive bytes k = 64h + 16b .. +15 (one buffer_load_dwordx4):
+// bytes 0..7 feed MFMA step 2h, bytes 8..15 step 2h + 1.  The matching activation fragment is 16 contiguous bytes of
+// x, staged per k-group into LDS one phase at a time in fragment order.  int8 -> bf16 is exact (sign-extending byte
+// convert, keep the high half).  No per-group arithmetic: the float32 accumulators run over all of K and the epilogue
+// reproduces the reference's two roundings, bf16(acc) then bf16(t * scale).
+#include "e2h_common.h"
+
+namespace e2h {
+namespace {
+
+constexpr int kChunk = 128;             // k per pipeline chunk
+constexpr int kSteps = 4;               // MFMA steps per chunk
+constexpr int kPPR = kChunk / 8;        // 16-byte activation pieces per row per chunk
+constexpr int kFragBytes = 1024 + 64;   // one fragment block in LDS (+ pad)
+
+__device__ __forceinline__ uint32_t pack_bf16_pair_exact(float lo, float hi) {
+  return (__builtin_bit_cast(uint32_t, lo) >> 16) | (__builtin_bit_cast(uint32_t, hi) & 0xFFFF0000u);
+}
+
+__device__ __forceinline__ bf16x8_t bytes_to_bf16x8(uint32_t d0, uint32_t d1) {
+  u32x4_t u;
+  u[0] = pack_bf16_pair_exact(static_cast<float>(static_cast<int8_t>(d0)), static_cast<float>(static_cast<int8_t>(d0 >> 8)));
+  u[1] = pack_bf16_pair_exact(static_cast<float>(static_cast<int8_t>(d0 >> 16)), static_cast<float>(static_cast<int8_t>(d0 >> 24)));
+  u[2] = pack_bf16_pair_exact(static_cast<float>(static_cast<int8_t>(d1)), static_cast<float>(static_cast<int8_t>(d1 >> 8)));
+  u[3] = pack_bf16_pair_exact(static_cast<float>(static_cast<int8_t>(d1 >> 16)), static_cast<float>(static_cast<int8_t>(d1 >> 24)));
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+
+template <int MT, int T, int WN, int WK>
+struct Tuning8 {
+  static constexpr int NB = (MT >= 4 || T >= 2) ? 2 : 4;                       // ring of weight chunks (2 KB per tile each)
+  static constexpr int kChunkLds = MT * kSteps * kFragBytes;
+  static constexpr int kLdsBudget = (WK >= 4 ? 144 : 72) * 1024;
+  static constexpr int CPP = (WK * 2 * 4 * kChunkLds <= kLdsBudget) ? 4 : ((WK * 2 * 2 * kChunkLds <= kLdsBudget) ? 2 : 1);
+  static constexpr int XD = (NB + CPP - 1) / CPP;
+};
+
+template <int T>
+struct WeightRegs8 {
+  u32x4_t w[T][2];
+};
+
+template <int MT, int T, int WN, int WK>
+__global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
+                                                                      const uint16_t *__restrict__ scales, uint16_t *__restrict__ y,
+                                                                      float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket,
+                                                                      int M, int N, int K) {
+  typedef Tuning8<MT, T, WN, WK> Tune;
+  constexpr int NB = Tune::NB, PD = NB - 1, CPP = Tune::CPP, XD = Tune::XD;
+  constexpr int U = NB > CPP * XD ? NB : CPP * XD;
+  constexpr int kGroupThreads = WN * 64;
+  constexpr int kPieces = 16 * MT * kPPR;
+  constexpr int kPhasePieces = CPP * kPieces;
+  constexpr int kPiecesPerThread = (kPhasePieces + kGroupThreads - 1) / kGroupThreads;
+  constexpr int kBufBytes = MT * kSteps * kFragBytes;
+  constexpr int kStageBytes = CPP * kBufBytes;
+  constexpr int kSlots = T * MT * 4;
+  constexpr int kXBytes = WK * 2 * kStageBytes;
+  constexpr int kRedBytes = (WK - 1) * WN * kSlots * 64 * 4;
+  constexpr int kLdsBytes = kXBytes > kRedBytes ? kXBytes : kRedBytes;
+
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+  __shared__ unsigned s_ticket;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_n = wave % WN;
+  const int kg = wave / WN;
+  const int tid_g = tid % kGroupThreads;
+  const int c = lane & 15;
+  const int b = lane >> 4;
+  const int nchunks = K / kChunk;
+  const int S = gridDim.y;
+  const int ks = blockIdx.y;
+  const int C0 = static_cast<int>((static_cast<long long>(nchunks) * ks) / S);
+  const int C1 = static_cast<int>((static_cast<long long>(nchunks) * (ks + 1)) / S);
+  const int c0 = C0 + ((C1 - C0) * kg) / WK;
+  const int c1 = C0 + ((C1 - C0) * (kg + 1)) / WK;
+  const int nloc = c1 - c0;
+  const int nloc_max = (C1 - C0 + WK - 1) / WK;
+  const int tile16_0 = (blockIdx.x * WN + wave_n) * T;
+  const int m_base = blockIdx.z * (16 * MT);
+  uint8_t *const xlds = lds + kg * (2 * kStageBytes);
+
+  uint32_t wlane[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    int n = 16 * (tile16_0 + t) + c;
+    n = n < N ? n : N - 1;
+    wlane[t] = static_cast<uint32_t>(static_cast<size_t>(n) * K + 16 * b);
+  }
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(q, static_cast<uint32_t>(static_cast<size_t>(N) * K));
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
+
+  auto load_weights = [&](WeightRegs8<T> &r, int ci) {
+    const uint32_t so = static_cast<uint32_t>(ci) * kChunk;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      r.w[t][0] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[t], so, 2);
+      r.w[t][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[t], so + 64, 2);
+    }
+  };
+
+  // activation staging: piece `within` (0..15) of a row's 128-wide chunk covers k = 8*within .. +7, which is the
+  // fragment of lane block b = (within % 8) / 2 in MFMA step 2 * (within / 8) + within % 2
+  uint32_t xsrc[kPiecesPerThread];
+  int xdst[kPiecesPerThread];
+  int xq[kPiecesPerThread];
+#pragma unroll
+  for (int i = 0; i < kPiecesPerThread; ++i) {
+    const int p = tid_g + i * kGroupThreads;
+    const int qc = (p / kPieces) < CPP ? (p / kPieces) : CPP - 1;
+    const int pc = p % kPieces;
+    int row = pc / kPPR;
+    const int within = pc % kPPR;
+    const int s = 2 * (within >> 3) + (within & 1), bb = (within & 7) >> 1;
+    xq[i] = qc;
+    xdst[i] = qc * kBufBytes + ((row >> 4) * kSteps + s) * kFragBytes + (bb * 16 + (row & 15)) * 16;
+    row += m_base;
+    row = row < M ? row : M - 1;
+    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + within * 8) * 2);
+  }
+  auto chunk_at = [&](int i) {
+    const int ci = c0 + (i < nloc ? i : nloc - 1);
+    return ci < C0 ? C0 : ci;
+  };
+  auto load_x = [&](u32x4_t (&r)[kPiecesPerThread], int phase) {
+#pragma unroll
+    for (int i = 0; i < kPiecesPerThread; ++i)
+      if (kPhasePieces % kGroupThreads == 0 || tid_g + i * kGroupThreads < kPhasePieces)
+        r[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(chunk_at(phase * CPP + xq[i])) * (kChunk * 2), 0);
+  };
+  auto store_x = [&](const u32x4_t (&r)[kPiecesPerThread], int parity) {
+    uint8_t *buf = xlds + (parity & 1) * kStageBytes;
+#pragma unroll
+    for (int i = 0; i < kPiecesPerThread; ++i)
+      if (kPhasePieces % kGroupThreads == 0 || tid_g + i * kGroupThreads < kPhasePieces)
+        *reinterpret_cast<u32x4_t *>(buf + xdst[i]) = r[i];
+  };
+
+  f32x4_t acc[T][MT];
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  auto compute_chunk = [&](const WeightRegs8<T> &r, int parity, int qc, uint32_t live) {
+    const uint8_t *buf = xlds + (parity & 1) * kStageBytes + qc * kBufBytes + lane * 16;
+    bf16x8_t xf[MT][kSteps];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) xf[mt][s] = *reinterpret_cast<const bf16x8_t *>(buf + (mt * kSteps + s) * kFragBytes);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // live == 0 (padding iteration): zero weights contribute nothing
+        const bf16x8_t w0 = bytes_to_bf16x8(r.w[t][h][0] & live, r.w[t][h][1] & live);
+        const bf16x8_t w1 = bytes_to_bf16x8(r.w[t][h][2] & live, r.w[t][h][3] & live);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][2 * h], w0, acc[t][mt], 0, 0, 0);
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][2 * h + 1], w1, acc[t][mt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  WeightRegs8<T> ring[NB];
+  u32x4_t xstage[XD][kPiecesPerThread];
+  if (C1 > C0) {
+#pragma unroll
+    for (int d = 0; d < XD; ++d) load_x(xstage[d], d);
+#pragma unroll
+    for (int i = 0; i < PD; ++i) load_weights(ring[i], chunk_at(i));
+    store_x(xstage[0], 0);
+    lds_barrier();
+    for (int base = 0; base < nloc_max; base += U) {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const int i = base + j;
+        const int phase = i / CPP;
+        const uint32_t live = i < nloc ? 0xFFFFFFFFu : 0u;
+        if (j % CPP == 0) load_x(xstage[(j / CPP) % XD], phase + XD);
+        load_weights(ring[(j + PD) % NB], chunk_at(i + PD));
+        compute_chunk(ring[j % NB], phase, j % CPP, live);
+        if (j % CPP == CPP - 1) {
+          store_x(xstage[(j / CPP + 1) % XD], phase + 1);
+          lds_barrier();
+        }
+      }
+    }
+  }
+
+  if constexpr (WK > 1) {
+    float *red = reinterpret_cast<float *>(lds);
+    if (kg > 0) {
+      float *mine = red + (static_cast<size_t>(kg - 1) * WN + wave_n) * kSlots * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) mine[((t * MT + mt) * 4 + r) * 64] = acc[t][mt][r];
+    }
+    lds_barrier();
+    if (kg == 0) {
+#pragma unroll
+      for (int g2 = 1; g2 < WK; ++g2) {
+        const float *other = red + (static_cast<size_t>(g2 - 1) * WN + wave_n) * kSlots * 64 + lane;
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[t][mt][r] += other[((t * MT + mt) * 4 + r) * 64];
+      }
+    }
+  }
+
+  if (S > 1) {
+    const size_t tile_floats = static_cast<size_t>(WN) * kSlots * 64;
+    const size_t wg_tile = static_cast<size_t>(blockIdx.z) * gridDim.x + blockIdx.x;
+    if (kg == 0) {
+      float *mine = ws_partial + (wg_tile * S + ks) * tile_floats + static_cast<size_t>(wave_n) * kSlots * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            __hip_atomic_store(mine + ((t * MT + mt) * 4 + r) * 64, acc[t][mt][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(ws_ticket + wg_tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != static_cast<unsigned>(S - 1)) return;
+    if (tid == 0) __hip_atomic_store(ws_ticket + wg_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (kg == 0) {
+      const float *all = ws_partial + wg_tile * S * tile_floats + static_cast<size_t>(wave_n) * kSlots * 64 + lane;
+      for (int s2 = 0; s2 < S; ++s2) {
+        float v[kSlots];
+#pragma unroll
+        for (int slot = 0; slot < kSlots; ++slot)
+          v[slot] = __hip_atomic_load(all + s2 * tile_floats + slot * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int slot = (t * MT + mt) * 4 + r;
+              acc[t][mt][r] = s2 == 0 ? v[slot] : acc[t][mt][r] + v[slot];
+            }
+      }
+    }
+  }
+  if (kg != 0) return;
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const int n = 16 * (tile16_0 + t) + c;
+    const float scale = bf16_to_f32(scales[n < N ? n : N - 1]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m_base + 16 * mt + 4 * b + r;
+        if (n < N && m < M) {
+          const float lin = bf16_round(acc[t][mt][r]);                              // F.linear output in bfloat16
+          y[static_cast<size_t>(m) * N + n] = f32_to_bf16_rne(lin * scale);        // * self.scales
+        }
+      }
+  }
+}
+
+struct Args8 {
+  const uint16_t *x;
+  const int8_t *q;
+  const uint16_t *scales;
+  uint16_t *y;
+  float *ws_partial;
+  unsigned *ws_ticket;
+  int M, N, K, S;
+  hipStream_t stream;
+};
+
+template <int MT, int T, int WN, int WK>
+int launch8(const Args8 &a) {
+  const int tiles16 = (a.N + 15) / 16;
+  dim3 grid((tiles16 + WN * T - 1) / (WN * T), a.S, (a.M + 16 * MT - 1) / (16 * MT));
+  hipLaunchKernelGGL((int8_stream_mm_kernel<MT, T, WN, WK>), grid, dim3(64 * WN * WK), 0, a.stream, a.x, a.q, a.scales, a.y,
+                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K);
+  return launch_status();
+}
+
+constexpr size_t kTicketBytes8 = 64 * 1024;
+constexpr int kCUs8 = 256;
+
+}  // namespace
+
+// Streaming int8 matmul; the caller has checked pointers and that K % 128 == 0 with 16-byte aligned x and q.
+int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int M, int N, int K, void *workspace,
+                   int64_t workspace_bytes, hipStream_t stream) {
+  Args8 a;
+  a.q = q; a.scales = scales; a.N = N; a.K = K; a.stream = stream;
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const int m_chunks = (M + 16 * mt - 1) / (16 * mt);
+  const int tiles16 = (N + 15) / 16;
+  const int nchunks = K / kChunk;
+  const bool have_ws = workspace && workspace_bytes >= static_cast<int64_t>(kTicketBytes8) + (int64_t{1} << 20);
+  int t = 1, wk = 2, s = 1;
+  if (mt == 4) {
+    wk = 1;
+    t = (static_cast<long long>((tiles16 + 7) / 8) * m_chunks >= kCUs8) ? 2 : 1;
+  } else {
+    const int blocks = ((tiles16 + 3) / 4) * m_chunks;
+    if (have_ws)
+      while (s < 4 && blocks * s < (3 * kCUs8) / 4 && nchunks / (2 * s * wk) >= 4) s *= 2;
+  }
+  if (options().int8_rows_per_wave == 16 || options().int8_rows_per_wave == 32) t = options().int8_rows_per_wave / 16;
+  if (options().int8_k_groups == 1 || options().int8_k_groups == 2) wk = options().int8_k_groups;
+  if (options().int8_k_slices > 0) s = options().int8_k_slices;
+  if (mt == 4) wk = 1;
+  if (s > nchunks) s = nchunks;
+  const int n_blocks = (tiles16 + 4 * t - 1) / (4 * t);
+  if (s > 1) {
+    const int64_t tile_floats = static_cast<int64_t>(4) * t * mt * 4 * 64;
+    const int64_t need = static_cast<int64_t>(kTicketBytes8) + static_cast<int64_t>(n_blocks) * m_chunks * s * tile_floats * 4;
+    if (!have_ws || need > workspace_bytes || static_cast<int64_t>(n_blocks) * m_chunks * 4 > static_cast<int64_t>(kTicketBytes8)) s = 1;
+  }
+  a.S = s;
+  a.ws_ticket = reinterpret_cast<unsigned *>(workspace);
+  a.ws_partial = workspace ? reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + kTicketBytes8) : nullptr;
+  const int64_t rows_by_bytes = ((int64_t{1} << 32) - 1) / (2 * static_cast<int64_t>(K));
+  const int64_t rows_by_grid = int64_t{65535} * 16 * mt;
+  int64_t max_rows = rows_by_bytes < rows_by_grid ? rows_by_bytes : rows_by_grid;
+  max_rows -= max_rows % (16 * mt);
+  if (max_rows < 16 * mt) return E2H_ERR_BAD_SHAPE;
+  for (int64_t m0 = 0; m0 < M; m0 += max_rows) {
+    a.x = x + m0 * K;
+    a.y = y + m0 * N;
+    a.M = static_cast<int>(M - m0 < max_rows ? M - m0 : max_rows);
+    int rc;
+    if (mt == 1) rc = t == 2 ? (wk == 2 ? launch8<1, 2, 4, 2>(a) : launch8<1, 2, 4, 1>(a)) : (wk == 2 ? launch8<1, 1, 4, 2>(a) : launch8<1, 1, 4, 1>(a));
+    else if (mt == 2) rc = t == 2 ? (wk == 2 ? launch8<2, 2, 4, 2>(a) : launch8<2, 2, 4, 1>(a)) : (wk == 2 ? launch8<2, 1, 4, 2>(a) : launch8<2, 1, 4, 1>(a));
+    else rc = t == 2 ? launch8<4, 2, 4, 1>(a) : launch8<4, 1, 4, 1>(a);
+    if (rc != E2H_OK) return rc;
+  }
+  return E2H_OK;
+}
+
+}  // namespace e2h

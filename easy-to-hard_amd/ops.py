@@ -91,7 +91,8 @@ def _int8_mm_impl(x, q, scales):
     y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     if m == 0:
         return y
-    rc = _lib_for(x).e2h_int8_mm(_ptr(x), _ptr(q), _ptr(scales), _ptr(y), m, n, k, _stream(x))
+    ws = _workspace(x.device)
+    rc = _lib_for(x).e2h_int8_mm(_ptr(x), _ptr(q), _ptr(scales), _ptr(y), m, n, k, _ptr(ws), ws.numel(), _stream(x))
     _lib.check(rc, "e2h_int8_mm")
     return y
 

@@ -38,7 +38,8 @@ extern "C" {
 int e2h_abi_version(void);
 const char *e2h_status_string(int status);
 
-/* Tuning knobs for experiments: name in {"int4_rows_per_wave", "int4_k_slices", "int8_rows_per_wave", "x_transpose"};
+/* Tuning knobs for experiments: launch-geometry overrides such as "int4_rows_per_wave", "int4_k_slices", "int4_k_groups",
+ * "int4_col_waves", "int8_rows_per_wave", "int8_k_groups", "int8_k_slices", "int8_force_generic";
  * value 0 restores the built-in heuristic.  Not thread safe; set before launching. */
 int e2h_set_option(const char *name, int value);
 
@@ -61,9 +62,10 @@ int e2h_int8_quantize_per_channel(const void *w, int w_is_bf16, int8_t *q, float
 /* WeightOnlyInt8Linear.forward, reference :428-429:  y = F.linear(x, weight.to(bf16)) * scales.
  *   x [m, k] bf16, q [n, k] int8, scales [n] bf16, y [m, n] bf16.  float32 accumulation; the result
  *   is rounded to bfloat16 before and after the multiplication by the scale, as in the reference.
- * Any m >= 1, n >= 1, k >= 1. */
+ * Any m >= 1, n >= 1, k >= 1 (k % 128 == 0 with 16-byte aligned x and q takes the streaming kernel).
+ * workspace / workspace_bytes: optional scratch as for e2h_int4_mm (NULL / 0 allowed). */
 int e2h_int8_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int64_t m,
-                int64_t n, int64_t k, void *stream);
+                int64_t n, int64_t k, void *workspace, int64_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------------------------------
  * int4, group-wise asymmetric

@@ -48,8 +48,8 @@ def test_argument_validation_returns_codes_without_launching():
     assert lib.e2h_int4_mm(p, p, p, p, 1, 8, 192, 128, 8, None, 0, None) == -3   # k % g != 0
     assert lib.e2h_int4_mm(p, p, p, p, 1, 8, 64, 32, 8, None, 0, None) == -4     # k % (16*ikt) != 0
     assert lib.e2h_int4_mm(ctypes.c_void_p(4098), p, p, p, 1, 8, 128, 128, 8, None, 0, None) == -5
-    assert lib.e2h_int8_mm(p, null, p, p, 1, 8, 128, None) == -1
-    assert lib.e2h_int8_mm(p, p, p, p, 1, 0, 128, None) == -2
+    assert lib.e2h_int8_mm(p, null, p, p, 1, 8, 128, None, 0, None) == -1
+    assert lib.e2h_int8_mm(p, p, p, p, 1, 0, 128, None, 0, None) == -2
     assert lib.e2h_int4_pack(p, p, 12, 128, 8, None) == -2
     assert lib.e2h_int4_pack(p, p, 8, 128, 5, None) == -4
     assert lib.e2h_int4_pack(p, p, 8, 64, 8, None) == -4
