@@ -5,7 +5,7 @@ no fallback implementation behind these entry points.
 """
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 
 from ._build import LIB_PATH, build_library
 
@@ -27,6 +27,10 @@ _SIGNATURES = {
     "e2h_int4_dequantize_codes": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int, _P]),
     "e2h_int4_mm": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P, c_int64, _P]),
     "e2h_workspace_bytes": (c_int64, []),
+    "e2h_decode_attention": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, _P]),
+    "e2h_rmsnorm": (c_int, [_P, _P, _P, c_int64, c_int64, c_float, _P]),
+    "e2h_rope_kv_write": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
+    "e2h_silu_mul": (c_int, [_P, _P, _P, c_int64, _P]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

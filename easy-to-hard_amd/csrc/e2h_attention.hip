@@ -1,0 +1,316 @@
+// Decode-step kernels around the quantized linears (HBM-bound, one launch each per layer):
+//   e2h_decode_attention   single-query attention over the bf16 KV cache, reading only the live positions
+//   e2h_rmsnorm            RMSNorm with the reference's rounding points
+//   e2h_rope_kv_write      rotary embedding of q and k + write of k, v into the cache at input_pos
+//   e2h_silu_mul           silu(a) * b
+// They restate, for one new token per sequence, what the reference's model code does with stock ops
+// (models/model.py: KVCache.update :121-129, Attention.forward :310-349, RMSNorm :363-377, apply_rotary_emb
+// :400-412, FeedForward.forward :359-360; decode loop inference_generate.py:110-157).
+#include "e2h_common.h"
+
+namespace e2h {
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// decode attention: q [B, H, D], caches [Bmax, Hkv, S, D] bf16, out [B, H, D] bf16.
+// One workgroup (4 waves) per (b, kv head); the waves split the live positions, every wave keeps REP query heads
+// (the heads that share the kv head) so that each K / V row is loaded once.  Lane layout: LPP = D/8 lanes cover
+// one position (16 bytes each), a wave-wide load covers 64/LPP positions.  Online softmax in float32.
+// Visible positions: t <= pos, and if left_pad is given additionally (t >= left_pad[b] or t == pos)
+// (reference models/model.py:221-228).
+// ------------------------------------------------------------------------------------------------
+template <int D, int REP>
+__global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
+                                                               const uint16_t *__restrict__ vc, uint16_t *__restrict__ out,
+                                                               const int64_t *__restrict__ input_pos, const int64_t *__restrict__ left_pad,
+                                                               int H, int Hkv, int S, float scale) {
+  constexpr int LPP = D / 8;        // lanes per position
+  constexpr int PPL = 64 / LPP;     // positions per wave-wide load
+  constexpr int UNR = 4;            // loads in flight per wave
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int dg = lane % LPP;        // which 8 values of the head dimension
+  const int pg = lane / LPP;        // which position within a load
+  const int b = blockIdx.x / Hkv, hk = blockIdx.x % Hkv;
+  const int pos = static_cast<int>(input_pos[0]);
+  const int first = left_pad ? static_cast<int>(left_pad[b]) : 0;
+  const int n_live = pos + 1;
+
+  float qf[REP][8];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(q + (static_cast<size_t>(b) * H + hk * REP + r) * D + dg * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      qf[r][2 * i] = __builtin_bit_cast(float, raw[i] << 16) * scale;
+      qf[r][2 * i + 1] = __builtin_bit_cast(float, raw[i] & 0xFFFF0000u) * scale;
+    }
+  }
+  const size_t head_base = (static_cast<size_t>(b) * Hkv + hk) * S * D;
+  const uint16_t *kbase = kc + head_base + dg * 8;
+  const uint16_t *vbase = vc + head_base + dg * 8;
+
+  float m_run[REP], l_run[REP], acc[REP][8];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    m_run[r] = -1e30f;
+    l_run[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
+  }
+
+  // waves take interleaved tiles of UNR * PPL positions
+  for (int t0 = wave * (UNR * PPL); t0 < n_live; t0 += 4 * UNR * PPL) {
+    u32x4_t kr[UNR], vr[UNR];
+    int tpos[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      tpos[u] = t0 + u * PPL + pg;
+      const int tc = tpos[u] < n_live ? tpos[u] : n_live - 1;
+      kr[u] = *reinterpret_cast<const u32x4_t *>(kbase + static_cast<size_t>(tc) * D);
+      vr[u] = *reinterpret_cast<const u32x4_t *>(vbase + static_cast<size_t>(tc) * D);
+    }
+    float s[REP][UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      float kf[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        kf[2 * i] = __builtin_bit_cast(float, kr[u][i] << 16);
+        kf[2 * i + 1] = __builtin_bit_cast(float, kr[u][i] & 0xFFFF0000u);
+      }
+      const bool visible = tpos[u] < n_live && (tpos[u] >= first || tpos[u] == pos);
+#pragma unroll
+      for (int r = 0; r < REP; ++r) {
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d = __builtin_fmaf(qf[r][i], kf[i], d);
+#pragma unroll
+        for (int off = 1; off < LPP; off <<= 1) d += __shfl_xor(d, off);
+        s[r][u] = visible ? d : -1e30f;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+      float mx = s[r][0];
+#pragma unroll
+      for (int u = 1; u < UNR; ++u) mx = fmaxf(mx, s[r][u]);
+#pragma unroll
+      for (int off = LPP; off < 64; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+      const float m_new = fmaxf(m_run[r], mx);
+      const float corr = __expf(m_run[r] - m_new);
+      m_run[r] = m_new;
+      l_run[r] *= corr;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[r][i] *= corr;
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const float p = s[r][u] > -1e29f ? __expf(s[r][u] - m_new) : 0.f;
+        l_run[r] += p;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[r][2 * i] = __builtin_fmaf(p, __builtin_bit_cast(float, vr[u][i] << 16), acc[r][2 * i]);
+          acc[r][2 * i + 1] = __builtin_fmaf(p, __builtin_bit_cast(float, vr[u][i] & 0xFFFF0000u), acc[r][2 * i + 1]);
+        }
+      }
+    }
+  }
+
+  // combine the position groups of a wave, then the waves
+  __shared__ float sh_m[4][REP], sh_l[4][REP], sh_acc[4][REP][D];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    // l_run counts each position once per lane of its group (every lane of the group holds the same p): sum over groups
+    float l = l_run[r];
+#pragma unroll
+    for (int off = LPP; off < 64; off <<= 1) l += __shfl_xor(l, off);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float a = acc[r][i];
+#pragma unroll
+      for (int off = LPP; off < 64; off <<= 1) a += __shfl_xor(a, off);
+      acc[r][i] = a;
+    }
+    if (pg == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sh_acc[wave][r][dg * 8 + i] = acc[r][i];
+      if (dg == 0) {
+        sh_m[wave][r] = m_run[r];
+        sh_l[wave][r] = l;
+      }
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < REP * D; e += 256) {
+    const int r = e / D, d = e % D;
+    float m = sh_m[0][r];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) m = fmaxf(m, sh_m[w][r]);
+    float l = 0.f, a = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float c = __expf(sh_m[w][r] - m);
+      l += sh_l[w][r] * c;
+      a += sh_acc[w][r][d] * c;
+    }
+    out[(static_cast<size_t>(b) * H + hk * REP + r) * D + d] = f32_to_bf16_rne(a / l);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// RMSNorm (reference :363-377): bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w), float32 statistics. One wave per row.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
+                                                      uint16_t *__restrict__ y, int rows, int dim, float eps) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const uint16_t *xr = x + static_cast<size_t>(row) * dim;
+  float ss = 0.f;
+  for (int i = lane * 8; i < dim; i += 512) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = __builtin_bit_cast(float, raw[j] << 16), bq = __builtin_bit_cast(float, raw[j] & 0xFFFF0000u);
+      ss = __builtin_fmaf(a, a, ss);
+      ss = __builtin_fmaf(bq, bq, ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / static_cast<float>(dim) + eps);
+  uint16_t *yr = y + static_cast<size_t>(row) * dim;
+  for (int i = lane * 8; i < dim; i += 512) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+    const u32x4_t wr = *reinterpret_cast<const u32x4_t *>(w + i);
+    u32x4_t o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = bf16_round(__builtin_bit_cast(float, raw[j] << 16) * inv) * __builtin_bit_cast(float, wr[j] << 16);
+      const float bq = bf16_round(__builtin_bit_cast(float, raw[j] & 0xFFFF0000u) * inv) * __builtin_bit_cast(float, wr[j] & 0xFFFF0000u);
+      o[j] = static_cast<uint32_t>(f32_to_bf16_rne(a)) | (static_cast<uint32_t>(f32_to_bf16_rne(bq)) << 16);
+    }
+    *reinterpret_cast<u32x4_t *>(yr + i) = o;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// RoPE + KV write for one new token per sequence.  qkv [B, (H + 2 Hkv) * D] bf16 (rows ordered q | k | v),
+// freqs [S, D/2, 2] bf16 (cos, sin).  Writes q_out [B, H, D] (rotated) and the caches at input_pos.
+// Rotation of interleaved pairs in float32, rounded to bf16 (reference :400-412).
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ freqs,
+                                                            uint16_t *__restrict__ q_out, uint16_t *__restrict__ kc, uint16_t *__restrict__ vc,
+                                                            const int64_t *__restrict__ input_pos, int B, int H, int Hkv, int S, int D) {
+  const int pairs_per_row = (H + 2 * Hkv) * D / 2;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= B * pairs_per_row) return;
+  const int b = idx / pairs_per_row, p = idx % pairs_per_row;
+  const int head = (2 * p) / D, dpair = p % (D / 2);
+  const int pos = static_cast<int>(input_pos[0]);
+  const uint32_t raw = reinterpret_cast<const uint32_t *>(qkv)[idx];
+  const float x0 = __builtin_bit_cast(float, raw << 16), x1 = __builtin_bit_cast(float, raw & 0xFFFF0000u);
+  if (head < H + Hkv) {
+    const uint32_t f = reinterpret_cast<const uint32_t *>(freqs)[static_cast<size_t>(pos) * (D / 2) + dpair];
+    const float cs = __builtin_bit_cast(float, f << 16), sn = __builtin_bit_cast(float, f & 0xFFFF0000u);
+    // two separately rounded products and their difference / sum, as torch evaluates the expression in float32
+    const float r0 = x0 * cs - x1 * sn;
+    const float r1 = x1 * cs + x0 * sn;
+    const uint32_t o = static_cast<uint32_t>(f32_to_bf16_rne(r0)) | (static_cast<uint32_t>(f32_to_bf16_rne(r1)) << 16);
+    if (head < H) {
+      reinterpret_cast<uint32_t *>(q_out)[(static_cast<size_t>(b) * H + head) * (D / 2) + dpair] = o;
+    } else {
+      const int hk = head - H;
+      reinterpret_cast<uint32_t *>(kc)[((static_cast<size_t>(b) * Hkv + hk) * S + pos) * (D / 2) + dpair] = o;
+    }
+  } else {
+    const int hk = head - H - Hkv;
+    reinterpret_cast<uint32_t *>(vc)[((static_cast<size_t>(b) * Hkv + hk) * S + pos) * (D / 2) + dpair] = raw;
+  }
+}
+
+// silu(a) * b with torch's rounding points: bf16(bf16(silu(a)) * b)
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restrict__ a, const uint16_t *__restrict__ bq,
+                                                       uint16_t *__restrict__ y, int64_t n8) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n8) return;
+  const u32x4_t ra = reinterpret_cast<const u32x4_t *>(a)[idx];
+  const u32x4_t rb = reinterpret_cast<const u32x4_t *>(bq)[idx];
+  u32x4_t o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float a0 = __builtin_bit_cast(float, ra[j] << 16), a1 = __builtin_bit_cast(float, ra[j] & 0xFFFF0000u);
+    const float s0 = bf16_round(a0 / (1.0f + expf(-a0))), s1 = bf16_round(a1 / (1.0f + expf(-a1)));
+    const float y0 = s0 * __builtin_bit_cast(float, rb[j] << 16), y1 = s1 * __builtin_bit_cast(float, rb[j] & 0xFFFF0000u);
+    o[j] = static_cast<uint32_t>(f32_to_bf16_rne(y0)) | (static_cast<uint32_t>(f32_to_bf16_rne(y1)) << 16);
+  }
+  reinterpret_cast<u32x4_t *>(y)[idx] = o;
+}
+
+template <int D>
+int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
+                     const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
+  switch (rep) {
+    case 1: hipLaunchKernelGGL((decode_attention_kernel<D, 1>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 2: hipLaunchKernelGGL((decode_attention_kernel<D, 2>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 4: hipLaunchKernelGGL((decode_attention_kernel<D, 4>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 8: hipLaunchKernelGGL((decode_attention_kernel<D, 8>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    default: return E2H_ERR_BAD_SHAPE;
+  }
+  return launch_status();
+}
+
+}  // namespace
+}  // namespace e2h
+
+using namespace e2h;
+
+extern "C" int e2h_decode_attention(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
+                                    const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch, int64_t n_head,
+                                    int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale, void *stream) {
+  if (!q || !k_cache || !v_cache || !out || !input_pos) return E2H_ERR_NULL_POINTER;
+  if (batch < 1 || n_head < 1 || n_kv_head < 1 || n_head % n_kv_head != 0 || cache_len < 1 || batch * n_kv_head > INT32_MAX)
+    return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return E2H_ERR_MISALIGNED;
+  const int rep = static_cast<int>(n_head / n_kv_head);
+  dim3 grid(static_cast<unsigned>(batch * n_kv_head));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (head_dim == 128)
+    return launch_attention<128>(rep, grid, s, q, k_cache, v_cache, out, input_pos, left_pad_mask_pos, (int)n_head, (int)n_kv_head, (int)cache_len, scale);
+  if (head_dim == 64)
+    return launch_attention<64>(rep, grid, s, q, k_cache, v_cache, out, input_pos, left_pad_mask_pos, (int)n_head, (int)n_kv_head, (int)cache_len, scale);
+  return E2H_ERR_BAD_SHAPE;
+}
+
+extern "C" int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream) {
+  if (!x || !weight || !y) return E2H_ERR_NULL_POINTER;
+  if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return E2H_ERR_MISALIGNED;
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), x, weight, y,
+                     static_cast<int>(rows), static_cast<int>(dim), eps);
+  return launch_status();
+}
+
+extern "C" int e2h_rope_kv_write(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache,
+                                 const int64_t *input_pos, int64_t batch, int64_t n_head, int64_t n_kv_head, int64_t cache_len,
+                                 int64_t head_dim, void *stream) {
+  if (!qkv || !freqs_cis || !q_out || !k_cache || !v_cache || !input_pos) return E2H_ERR_NULL_POINTER;
+  if (batch < 1 || n_head < 1 || n_kv_head < 1 || head_dim < 2 || head_dim % 2 != 0) return E2H_ERR_BAD_SHAPE;
+  const int64_t pairs = batch * (n_head + 2 * n_kv_head) * head_dim / 2;
+  if (pairs > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), qkv,
+                     freqs_cis, q_out, k_cache, v_cache, input_pos, (int)batch, (int)n_head, (int)n_kv_head, (int)cache_len, (int)head_dim);
+  return launch_status();
+}
+
+extern "C" int e2h_silu_mul(const uint16_t *a, const uint16_t *b, uint16_t *y, int64_t n, void *stream) {
+  if (!a || !b || !y) return E2H_ERR_NULL_POINTER;
+  if (n < 8 || n % 8 != 0) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(a) || !aligned16(b) || !aligned16(y)) return E2H_ERR_MISALIGNED;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3(static_cast<unsigned>((n / 8 + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), a, b, y, n / 8);
+  return launch_status();
+}

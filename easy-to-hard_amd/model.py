@@ -15,7 +15,16 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch import Tensor
 
+from . import ops
 from .quantize import find_multiple
+
+# When True (default) and the tensors are bf16 on the GPU, RMSNorm, SiLU*mul and -- for single-token steps with
+# a KV cache -- RoPE + cache write + attention run as this package's fused kernels instead of chains of stock ops.
+FUSED_DECODE = True
+
+
+def _fusable(t: Tensor) -> bool:
+    return FUSED_DECODE and t.is_cuda and t.dtype == torch.bfloat16 and not torch.compiler.is_compiling()
 
 
 @dataclass
@@ -93,6 +102,8 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(dim))
 
     def forward(self, x: Tensor) -> Tensor:
+        if _fusable(x) and self.weight.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0:
+            return ops.rmsnorm(x, self.weight, self.eps)
         xf = x.float()
         normed = xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + self.eps)
         return normed.to(dtype=x.dtype) * self.weight
@@ -124,6 +135,8 @@ class Attention(nn.Module):
         self.wqkv = nn.Linear(config.dim, total_head_dim, bias=False)  # rows ordered [q | k | v]
         self.wo = nn.Linear(config.dim, config.dim, bias=False)
         self.kv_cache = None
+        self.freqs_table = None        # full (cos, sin) table, set by Transformer.setup_caches
+        self.left_pad_mask_pos = None  # per-step padding mask positions, set by Transformer.forward
         self.n_head = config.n_head
         self.head_dim = config.head_dim
         self.n_local_heads = config.n_local_heads
@@ -137,10 +150,22 @@ class Attention(nn.Module):
             parts = [state_dict.pop(prefix + n + ".weight") for n in ("wq", "wk", "wv")]
             state_dict[prefix + "wqkv.weight"] = torch.cat(parts)
 
-    def forward(self, x: Tensor, freqs_cis: Tensor, mask: Optional[Tensor], input_pos: Optional[Tensor] = None,
+    def can_fuse_decode(self, x: Tensor, fully_causal: bool) -> bool:
+        return (x.shape[1] == 1 and not fully_causal and self.kv_cache is not None and _fusable(x)
+                and self.freqs_table is not None and self.head_dim in (64, 128)
+                and (self.n_head // self.n_local_heads) in (1, 2, 4, 8))
+
+    def forward(self, x: Tensor, freqs_cis: Optional[Tensor], mask: Optional[Tensor], input_pos: Optional[Tensor] = None,
                 fully_causal: bool = False) -> Tensor:
         bsz, seqlen, _ = x.shape
         kv_size = self.n_local_heads * self.head_dim
+        if self.can_fuse_decode(x, fully_causal):
+            # one new token per sequence: RoPE + cache write in one kernel, then attention over the live positions only
+            qkv = self.wqkv(x).view(bsz, -1)
+            q = ops.rope_kv_write(qkv, self.freqs_table, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos,
+                                  self.n_head, self.n_local_heads, self.head_dim)
+            y = ops.decode_attention(q, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, self.left_pad_mask_pos)
+            return self.wo(y.view(bsz, 1, self.dim))
         q, k, v = self.wqkv(x).split([self.dim, kv_size, kv_size], dim=-1)
         q = apply_rotary_emb(q.view(bsz, seqlen, self.n_head, self.head_dim), freqs_cis).transpose(1, 2)
         k = apply_rotary_emb(k.view(bsz, seqlen, self.n_local_heads, self.head_dim), freqs_cis).transpose(1, 2)
@@ -167,7 +192,10 @@ class FeedForward(nn.Module):
         self.w2 = nn.Linear(config.intermediate_size, config.dim, bias=False)
 
     def forward(self, x: Tensor) -> Tensor:
-        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+        a, b = self.w1(x), self.w3(x)
+        if _fusable(a) and a.numel() % 8 == 0:
+            return self.w2(ops.silu_mul(a, b))
+        return self.w2(F.silu(a) * b)
 
 
 class TransformerBlock(nn.Module):
@@ -218,6 +246,8 @@ class Transformer(nn.Module):
             )
         self.kv_cache_enabled = kv_cache
         self.freqs_cis = precompute_freqs_cis(max(cfg.block_size, max_seq_length), cfg.head_dim, cfg.rope_base, device=device)
+        for blk in self.layers:
+            blk.attention.freqs_table = self.freqs_cis
         self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
         self.self_mask = torch.eye(max_seq_length, dtype=torch.bool, device=device)
 
@@ -226,15 +256,18 @@ class Transformer(nn.Module):
         """idx [B, S] token ids, input_pos [S] positions -> logits [B, S, vocab] (reference :212-248)."""
         assert self.freqs_cis is not None, "Caches must be initialized first"
         assert not (fully_causal and left_pad_mask_pos is not None), "Invalid mask"
+        for blk in self.layers:
+            blk.attention.left_pad_mask_pos = left_pad_mask_pos
+        x = self.tok_embeddings(idx)
         mask = None
-        if not fully_causal:
+        fused_step = self.layers[0].attention.can_fuse_decode(x, fully_causal)
+        if not fully_causal and not fused_step:
             mask = self.causal_mask[None, None, input_pos]
             if left_pad_mask_pos is not None:
                 visible = torch.arange(mask.size(-1), device=mask.device).view(1, -1) >= left_pad_mask_pos.view(-1, 1)
                 mask = torch.logical_and(mask, visible[:, None, None, :])
                 mask = torch.logical_or(mask, self.self_mask[None, None, input_pos])
-        x = self.tok_embeddings(idx)
-        freqs_cis = self.freqs_cis[input_pos].to(dtype=x.dtype)
+        freqs_cis = None if fused_step else self.freqs_cis[input_pos].to(dtype=x.dtype)
         for layer in self.layers:
             x = layer(x, input_pos, freqs_cis, mask, fully_causal)
         return self.output(self.norm(x))

@@ -305,3 +305,65 @@ def int4_mm_direct(x, packed, groupsize, scales_and_zeros):
 
 def int8_mm_direct(x, q, scales):
     return _int8_mm_impl(x, q, scales)
+
+
+# ---------------------------------------------------------------------------------------------
+# decode-step kernels around the linears (harness side; stock torch ops are the fallback only off the GPU)
+# ---------------------------------------------------------------------------------------------
+
+
+def rmsnorm(x, weight, eps):
+    """bf16 [..., dim] -> bf16, reference RMSNorm rounding (models/model.py:363-377)."""
+    _need_gpu(x, weight)
+    assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    dim = x.shape[-1]
+    rc = _lib_for(x).e2h_rmsnorm(_ptr(x), _ptr(weight), _ptr(y), x.numel() // dim, dim, float(eps), _stream(x))
+    _lib.check(rc, "e2h_rmsnorm")
+    return y
+
+
+def silu_mul(a, b):
+    """bf16(bf16(silu(a)) * b), same shape."""
+    _need_gpu(a, b)
+    assert a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and a.shape == b.shape
+    a, b = a.contiguous(), b.contiguous()
+    y = torch.empty_like(a)
+    rc = _lib_for(a).e2h_silu_mul(_ptr(a), _ptr(b), _ptr(y), a.numel(), _stream(a))
+    _lib.check(rc, "e2h_silu_mul")
+    return y
+
+
+def rope_kv_write(qkv, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head, head_dim):
+    """qkv bf16 [B, (H + 2 Hkv) * D] of one new token per sequence -> rotated q [B, H, D]; rotated k and v are
+    written into the caches [Bmax, Hkv, S, D] at input_pos (int64 device tensor with one element)."""
+    _need_gpu(qkv, freqs_cis, k_cache, v_cache, input_pos)
+    assert qkv.dtype == torch.bfloat16 and freqs_cis.dtype == torch.bfloat16 and input_pos.dtype == torch.int64
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and freqs_cis.is_contiguous()
+    qkv = qkv.contiguous()
+    bsz = qkv.shape[0]
+    assert qkv.shape[1] == (n_head + 2 * n_kv_head) * head_dim and k_cache.shape[1] == n_kv_head and k_cache.shape[3] == head_dim
+    q = torch.empty((bsz, n_head, head_dim), dtype=torch.bfloat16, device=qkv.device)
+    rc = _lib_for(qkv).e2h_rope_kv_write(_ptr(qkv), _ptr(freqs_cis), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(input_pos), bsz,
+                                         n_head, n_kv_head, k_cache.shape[2], head_dim, _stream(qkv))
+    _lib.check(rc, "e2h_rope_kv_write")
+    return q
+
+
+def decode_attention(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, scale=None):
+    """q bf16 [B, H, D] against caches [Bmax, Hkv, S, D] up to and including input_pos -> bf16 [B, H, D]."""
+    _need_gpu(q, k_cache, v_cache, input_pos)
+    assert q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and input_pos.dtype == torch.int64
+    q = q.contiguous()
+    bsz, n_head, head_dim = q.shape
+    if scale is None:
+        scale = head_dim ** -0.5
+    lp = None
+    if left_pad_mask_pos is not None:
+        lp = left_pad_mask_pos.to(torch.int64).contiguous()
+    out = torch.empty_like(q)
+    rc = _lib_for(q).e2h_decode_attention(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(input_pos), _ptr(lp) if lp is not None else None,
+                                          bsz, n_head, k_cache.shape[1], k_cache.shape[2], head_dim, float(scale), _stream(q))
+    _lib.check(rc, "e2h_decode_attention")
+    return out

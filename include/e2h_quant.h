@@ -130,6 +130,36 @@ int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales
 /* Recommended size in bytes of the workspace accepted by the matmul entry points (no reference counterpart). */
 int64_t e2h_workspace_bytes(void);
 
+/* ------------------------------------------------------------------------------------------------
+ * Decode-step kernels around the quantized linears (callers of the hot path; stock-op equivalents in the
+ * reference's models/model.py).  bf16 everywhere, float32 arithmetic inside.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Single-query attention over the KV cache, reference Attention.forward models/model.py:310-349 with
+ * KVCache :112-129 and the mask of Transformer.forward :221-228, for one new token per sequence.
+ *   q [batch, n_head, head_dim]; k_cache, v_cache [>= batch, n_kv_head, cache_len, head_dim]; out [batch, n_head, head_dim].
+ *   input_pos: device pointer to the position of the new token (positions 0..pos are attended);
+ *   left_pad_mask_pos: NULL or device [batch]: positions below it are masked except the new token itself.
+ * head_dim in {64, 128}; n_head / n_kv_head in {1, 2, 4, 8}. */
+int e2h_decode_attention(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
+                         const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch,
+                         int64_t n_head, int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale,
+                         void *stream);
+
+/* RMSNorm, reference models/model.py:363-377: y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * weight). x, y [rows, dim]. */
+int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *y, int64_t rows, int64_t dim, float eps,
+                void *stream);
+
+/* apply_rotary_emb (reference :400-412) on the q and k parts of a fused qkv row + KVCache.update (:121-129) for
+ * one new token per sequence.  qkv [batch, (n_head + 2 n_kv_head) * head_dim]; freqs_cis [positions, head_dim/2, 2]
+ * bf16 (cos, sin); q_out [batch, n_head, head_dim]; caches as above, written at *input_pos. */
+int e2h_rope_kv_write(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache,
+                      uint16_t *v_cache, const int64_t *input_pos, int64_t batch, int64_t n_head,
+                      int64_t n_kv_head, int64_t cache_len, int64_t head_dim, void *stream);
+
+/* F.silu(a) * b with bf16 rounding after each op (reference FeedForward.forward :359-360). n elements, n % 8 == 0. */
+int e2h_silu_mul(const uint16_t *a, const uint16_t *b, uint16_t *y, int64_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

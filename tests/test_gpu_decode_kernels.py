@@ -1,0 +1,100 @@
+"""GPU checks of the decode-step kernels around the linears (RMSNorm, SiLU*mul, RoPE + KV write, single-query
+attention) against the stock torch ops the harness otherwise uses, through the C ABI."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import easy_to_hard_amd.model as model_mod
+from easy_to_hard_amd import ops
+from easy_to_hard_amd.generate import decode_one_token, prefill
+from easy_to_hard_amd.model import Transformer, apply_rotary_emb, init_random_, precompute_freqs_cis
+from tests.helpers import randn_bf16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_rmsnorm_matches_stock_ops():
+    for rows, dim in [(32, 4096), (5, 256), (1, 8192), (70, 512)]:
+        x = randn_bf16((rows, dim), std=1.5, seed=rows).to(DEV)
+        w = (1 + 0.1 * randn_bf16((dim,), seed=dim).float()).to(torch.bfloat16).to(DEV)
+        xf = x.float()
+        ref = (xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + 1e-5)).to(torch.bfloat16) * w
+        y = ops.rmsnorm(x, w, 1e-5)
+        # identical up to the summation order of mean(x^2): at most one bf16 ulp, almost always zero
+        assert torch.allclose(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+        assert (y == ref).float().mean() > 0.99
+
+
+def test_silu_mul_matches_stock_ops():
+    a = randn_bf16((32, 11008), std=2.0, seed=1).to(DEV)
+    b = randn_bf16((32, 11008), std=1.0, seed=2).to(DEV)
+    ref = F.silu(a) * b
+    y = ops.silu_mul(a, b)
+    assert torch.allclose(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+    assert (y == ref).float().mean() > 0.99
+
+
+@pytest.mark.parametrize("n_head,n_kv,d", [(32, 32, 128), (64, 8, 128), (4, 4, 64), (8, 2, 64)])
+def test_rope_kv_write_and_attention_match_stock_ops(n_head, n_kv, d):
+    bsz, s_max, pos = 3, 96, 41
+    gen = torch.Generator().manual_seed(n_head + d)
+    qkv = (torch.randn((bsz, (n_head + 2 * n_kv) * d), generator=gen)).to(torch.bfloat16).to(DEV)
+    kc = (torch.randn((bsz + 1, n_kv, s_max, d), generator=gen)).to(torch.bfloat16).to(DEV)
+    vc = (torch.randn((bsz + 1, n_kv, s_max, d), generator=gen)).to(torch.bfloat16).to(DEV)
+    freqs = precompute_freqs_cis(s_max, d, 10000, device=DEV)
+    input_pos = torch.tensor([pos], device=DEV)
+    # stock path
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    q, k, v = qkv.view(bsz, 1, -1).split([n_head * d, n_kv * d, n_kv * d], dim=-1)
+    fc = freqs[input_pos]
+    q_ref = apply_rotary_emb(q.view(bsz, 1, n_head, d), fc).transpose(1, 2)
+    k_rot = apply_rotary_emb(k.view(bsz, 1, n_kv, d), fc).transpose(1, 2)
+    kc_ref[:bsz].index_copy_(2, input_pos, k_rot)
+    vc_ref[:bsz].index_copy_(2, input_pos, v.view(bsz, 1, n_kv, d).transpose(1, 2))
+    # fused kernel
+    q_out = ops.rope_kv_write(qkv, freqs, kc, vc, input_pos, n_head, n_kv, d)
+    assert torch.equal(q_out, q_ref.squeeze(2))
+    assert torch.equal(kc, kc_ref) and torch.equal(vc, vc_ref)
+    # attention over positions 0..pos, with and without a left-padding mask
+    for left_pad in (None, torch.tensor([0, 7, 41], device=DEV)):
+        mask = (torch.arange(s_max, device=DEV) <= pos)[None, None, None, :]
+        if left_pad is not None:
+            vis = torch.arange(s_max, device=DEV).view(1, -1) >= left_pad.view(-1, 1)
+            mask = torch.logical_and(mask, vis[:, None, None, :])
+            mask = torch.logical_or(mask, (torch.arange(s_max, device=DEV) == pos)[None, None, None, :])
+        rep = n_head // n_kv
+        kk = kc_ref[:bsz].repeat_interleave(rep, dim=1).float()
+        vv = vc_ref[:bsz].repeat_interleave(rep, dim=1).float()
+        ref = F.scaled_dot_product_attention(q_ref.float(), kk, vv, attn_mask=mask).squeeze(2)
+        y = ops.decode_attention(q_out, kc, vc, input_pos, left_pad)
+        assert y.shape == (bsz, n_head, d)
+        err = (y.float() - ref).abs().max() / ref.abs().max()
+        assert err < 1e-2, err
+
+
+def test_fused_decode_step_matches_stock_decode_step():
+    model = Transformer.from_name("tiny-gqa-test")
+    init_random_(model, seed=5, std=0.05)
+    model = model.to(device=DEV, dtype=torch.bfloat16).eval()
+    bsz, t = 3, 9
+    prompt = torch.randint(0, 512, (bsz, t), generator=torch.Generator().manual_seed(2)).to(DEV)
+    logits = {}
+    for fused in (False, True):
+        model_mod.FUSED_DECODE = fused
+        try:
+            model.max_seq_length = -1
+            model.setup_caches(bsz, 32)
+            cur = prefill(model, prompt, torch.arange(0, t, device=DEV))
+            out = []
+            for i in range(4):
+                pos = torch.tensor([t + i], device=DEV)
+                lg = model(cur, pos)
+                out.append(lg[:, -1].float())
+                cur = torch.argmax(lg[:, -1].float(), dim=-1, keepdim=True)
+            logits[fused] = torch.stack(out)
+        finally:
+            model_mod.FUSED_DECODE = True
+    err = (logits[True] - logits[False]).abs().max() / logits[False].abs().max()
+    assert err < 2e-2, err
