@@ -29,6 +29,7 @@ _SIGNATURES = {
     "e2h_workspace_bytes": (c_int64, []),
     "e2h_decode_attention": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, _P]),
     "e2h_rmsnorm": (c_int, [_P, _P, _P, c_int64, c_int64, c_float, _P]),
+    "e2h_add_rmsnorm": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "e2h_rope_kv_write": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
     "e2h_silu_mul": (c_int, [_P, _P, _P, c_int64, _P]),
 }

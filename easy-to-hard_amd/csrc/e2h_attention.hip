@@ -163,17 +163,32 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *_
 }
 
 // ------------------------------------------------------------------------------------------------
-// RMSNorm (reference :363-377): bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w), float32 statistics. One wave per row.
+// RMSNorm (reference :363-377): bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w), float32 statistics.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
-                                                      uint16_t *__restrict__ y, int rows, int dim, float eps) {
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (row >= rows) return;
-  const uint16_t *xr = x + static_cast<size_t>(row) * dim;
+// One workgroup per row.  With `delta` the kernel first forms h = bf16(x + delta) (the residual add of
+// TransformerBlock.forward, reference :279-282), stores it to h_out and normalises h.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ delta,
+                                                      const uint16_t *__restrict__ w, uint16_t *__restrict__ h_out,
+                                                      uint16_t *__restrict__ y, int dim, float eps) {
+  const size_t row = blockIdx.x;
+  const uint16_t *xr = x + row * dim;
+  constexpr int kMaxPieces = 4;  // dim <= 256 * 8 * 4 = 8192 values are kept in registers, longer rows are re-read
+  u32x4_t keep[kMaxPieces];
   float ss = 0.f;
-  for (int i = lane * 8; i < dim; i += 512) {
-    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+  int np = 0;
+  for (int i = threadIdx.x * 8; i < dim; i += 2048, ++np) {
+    u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+    if (delta) {
+      const u32x4_t dr = *reinterpret_cast<const u32x4_t *>(delta + row * dim + i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a = __builtin_bit_cast(float, raw[j] << 16) + __builtin_bit_cast(float, dr[j] << 16);
+        const float bq = __builtin_bit_cast(float, raw[j] & 0xFFFF0000u) + __builtin_bit_cast(float, dr[j] & 0xFFFF0000u);
+        raw[j] = static_cast<uint32_t>(f32_to_bf16_rne(a)) | (static_cast<uint32_t>(f32_to_bf16_rne(bq)) << 16);
+      }
+      *reinterpret_cast<u32x4_t *>(h_out + row * dim + i) = raw;
+    }
+    if (np < kMaxPieces) keep[np] = raw;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float a = __builtin_bit_cast(float, raw[j] << 16), bq = __builtin_bit_cast(float, raw[j] & 0xFFFF0000u);
@@ -182,10 +197,16 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
     }
   }
   ss = wave_sum(ss);
+  __shared__ float part[4];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = (part[0] + part[1]) + (part[2] + part[3]);
   const float inv = rsqrtf(ss / static_cast<float>(dim) + eps);
-  uint16_t *yr = y + static_cast<size_t>(row) * dim;
-  for (int i = lane * 8; i < dim; i += 512) {
-    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+  const uint16_t *src = delta ? h_out + row * dim : xr;
+  uint16_t *yr = y + row * dim;
+  np = 0;
+  for (int i = threadIdx.x * 8; i < dim; i += 2048, ++np) {
+    const u32x4_t raw = np < kMaxPieces ? keep[np] : *reinterpret_cast<const u32x4_t *>(src + i);
     const u32x4_t wr = *reinterpret_cast<const u32x4_t *>(w + i);
     u32x4_t o;
 #pragma unroll
@@ -290,8 +311,18 @@ extern "C" int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *
   if (!x || !weight || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<unsigned>((rows + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), x, weight, y,
-                     static_cast<int>(rows), static_cast<int>(dim), eps);
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream), x, nullptr, weight, nullptr,
+                     y, static_cast<int>(dim), eps);
+  return launch_status();
+}
+
+extern "C" int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *weight, uint16_t *h_out, uint16_t *y,
+                               int64_t rows, int64_t dim, float eps, void *stream) {
+  if (!x || !delta || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
+  if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(delta) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream), x, delta, weight, h_out,
+                     y, static_cast<int>(dim), eps);
   return launch_status();
 }
 

@@ -207,7 +207,11 @@ class TransformerBlock(nn.Module):
         self.attention_norm = RMSNorm(config.dim, config.norm_eps)
 
     def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Optional[Tensor], fully_causal: bool = False) -> Tensor:
-        h = x + self.attention(self.attention_norm(x), freqs_cis, mask, input_pos, fully_causal)
+        attn = self.attention(self.attention_norm(x), freqs_cis, mask, input_pos, fully_causal)
+        if _fusable(x) and self.ffn_norm.weight.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0:
+            h, normed = ops.add_rmsnorm(x, attn, self.ffn_norm.weight, self.ffn_norm.eps)
+            return h + self.feed_forward(normed)
+        h = x + attn
         return h + self.feed_forward(self.ffn_norm(h))
 
 

@@ -324,6 +324,19 @@ def rmsnorm(x, weight, eps):
     return y
 
 
+def add_rmsnorm(x, delta, weight, eps):
+    """h = bf16(x + delta); returns (h, RMSNorm(h)) -- the residual add and the following norm in one kernel."""
+    _need_gpu(x, delta, weight)
+    assert x.dtype == torch.bfloat16 and delta.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape == delta.shape
+    x, delta = x.contiguous(), delta.contiguous()
+    h = torch.empty_like(x)
+    y = torch.empty_like(x)
+    dim = x.shape[-1]
+    rc = _lib_for(x).e2h_add_rmsnorm(_ptr(x), _ptr(delta), _ptr(weight), _ptr(h), _ptr(y), x.numel() // dim, dim, float(eps), _stream(x))
+    _lib.check(rc, "e2h_add_rmsnorm")
+    return h, y
+
+
 def silu_mul(a, b):
     """bf16(bf16(silu(a)) * b), same shape."""
     _need_gpu(a, b)

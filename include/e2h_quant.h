@@ -150,6 +150,11 @@ int e2h_decode_attention(const uint16_t *q, const uint16_t *k_cache, const uint1
 int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *y, int64_t rows, int64_t dim, float eps,
                 void *stream);
 
+/* Residual add + RMSNorm in one pass (TransformerBlock.forward, reference :279-282):
+ * h_out = bf16(x + delta), y = RMSNorm(h_out).  All [rows, dim]. */
+int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *weight, uint16_t *h_out,
+                    uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream);
+
 /* apply_rotary_emb (reference :400-412) on the q and k parts of a fused qkv row + KVCache.update (:121-129) for
  * one new token per sequence.  qkv [batch, (n_head + 2 n_kv_head) * head_dim]; freqs_cis [positions, head_dim/2, 2]
  * bf16 (cos, sin); q_out [batch, n_head, head_dim]; caches as above, written at *input_pos. */

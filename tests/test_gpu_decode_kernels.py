@@ -16,13 +16,27 @@ DEV = "cuda:0"
 
 
 def test_rmsnorm_matches_stock_ops():
-    for rows, dim in [(32, 4096), (5, 256), (1, 8192), (70, 512)]:
+    for rows, dim in [(32, 4096), (5, 256), (1, 8192), (70, 512), (2, 16384)]:
         x = randn_bf16((rows, dim), std=1.5, seed=rows).to(DEV)
         w = (1 + 0.1 * randn_bf16((dim,), seed=dim).float()).to(torch.bfloat16).to(DEV)
         xf = x.float()
         ref = (xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + 1e-5)).to(torch.bfloat16) * w
         y = ops.rmsnorm(x, w, 1e-5)
         # identical up to the summation order of mean(x^2): at most one bf16 ulp, almost always zero
+        assert torch.allclose(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+        assert (y == ref).float().mean() > 0.99
+
+
+def test_add_rmsnorm_matches_stock_ops():
+    for rows, dim in [(32, 4096), (3, 256), (2, 16384)]:
+        x = randn_bf16((rows, dim), std=1.5, seed=rows).to(DEV)
+        d = randn_bf16((rows, dim), std=0.7, seed=rows + 1).to(DEV)
+        w = (1 + 0.1 * randn_bf16((dim,), seed=dim).float()).to(torch.bfloat16).to(DEV)
+        h_ref = x + d
+        hf = h_ref.float()
+        ref = (hf * torch.rsqrt(torch.mean(hf * hf, dim=-1, keepdim=True) + 1e-5)).to(torch.bfloat16) * w
+        h, y = ops.add_rmsnorm(x, d, w, 1e-5)
+        assert torch.equal(h, h_ref)
         assert torch.allclose(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
         assert (y == ref).float().mean() > 0.99
 
