@@ -207,12 +207,26 @@ class TransformerBlock(nn.Module):
         self.attention_norm = RMSNorm(config.dim, config.norm_eps)
 
     def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Optional[Tensor], fully_causal: bool = False) -> Tensor:
-        attn = self.attention(self.attention_norm(x), freqs_cis, mask, input_pos, fully_causal)
+        return self._after_norm(x, self.attention_norm(x), input_pos, freqs_cis, mask, fully_causal)
+
+    def _after_norm(self, x, normed, input_pos, freqs_cis, mask, fully_causal):
+        attn = self.attention(normed, freqs_cis, mask, input_pos, fully_causal)
         if _fusable(x) and self.ffn_norm.weight.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0:
             h, normed = ops.add_rmsnorm(x, attn, self.ffn_norm.weight, self.ffn_norm.eps)
             return h + self.feed_forward(normed)
         h = x + attn
         return h + self.feed_forward(self.ffn_norm(h))
+
+    def forward_deferred(self, x: Tensor, delta: Optional[Tensor], input_pos, freqs_cis, mask, fully_causal: bool = False):
+        """Fused-path variant: `delta` is the previous block's feed-forward output that has not been added to the
+        residual stream yet; the add is folded into this block's first norm.  Returns (h, this block's pending delta)."""
+        if delta is None:
+            normed = ops.rmsnorm(x, self.attention_norm.weight, self.attention_norm.eps)
+        else:
+            x, normed = ops.add_rmsnorm(x, delta, self.attention_norm.weight, self.attention_norm.eps)
+        attn = self.attention(normed, freqs_cis, mask, input_pos, fully_causal)
+        h, normed2 = ops.add_rmsnorm(x, attn, self.ffn_norm.weight, self.ffn_norm.eps)
+        return h, self.feed_forward(normed2)
 
 
 class Transformer(nn.Module):
@@ -272,6 +286,12 @@ class Transformer(nn.Module):
                 mask = torch.logical_and(mask, visible[:, None, None, :])
                 mask = torch.logical_or(mask, self.self_mask[None, None, input_pos])
         freqs_cis = None if fused_step else self.freqs_cis[input_pos].to(dtype=x.dtype)
+        if _fusable(x) and x.shape[-1] % 8 == 0 and self.norm.weight.dtype == torch.bfloat16:
+            delta = None
+            for layer in self.layers:
+                x, delta = layer.forward_deferred(x, delta, input_pos, freqs_cis, mask, fully_causal)
+            _, normed = ops.add_rmsnorm(x, delta, self.norm.weight, self.norm.eps)
+            return self.output(normed)
         for layer in self.layers:
             x = layer(x, input_pos, freqs_cis, mask, fully_causal)
         return self.output(self.norm(x))
