@@ -109,10 +109,18 @@ struct Tuning {
 // WN = waves that share one activation stream and split the workgroup's columns; WK = number of k-groups
 // inside the workgroup (each group = WN waves with its own activation stream over a contiguous part of the
 // workgroup's K slice); the k-groups' accumulators are added through LDS at the end.
-template <int G, int IKT, int MT, int T, int WN, int WK>
+//
+// GATE: the two "tiles" of a wave are the same 16 columns of two weight matrices of equal shape (wp / sz and
+// wp2 / sz2, the gate and up projections of a feed-forward block); the epilogue writes
+// bf16(bf16(silu(bf16(gate))) * bf16(up)), the rounding points of  F.silu(w1(x)) * w3(x)  on bfloat16 tensors
+// (reference models/model.py:343-344).  Both products share one activation stream.
+template <int G, int IKT, int MT, int T, int WN, int WK, bool GATE = false>
 __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
+    const uint32_t *__restrict__ wp2, const uint32_t *__restrict__ sz2,
     uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K) {
+  static_assert(!GATE || T == 2, "gate mode pairs exactly two weight matrices");
+  constexpr int TC = GATE ? 1 : T;  // distinct column tiles per wave
   typedef Int4Geom<G, IKT> Geo;
   typedef WeightRegs<G, IKT, T> wregs_t;
   constexpr int kWavesN = WN;
@@ -155,7 +163,7 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   const int c1 = C0 + ((C1 - C0) * (kg + 1)) / WK;
   const int nloc = c1 - c0;
   const int nloc_max = (C1 - C0 + WK - 1) / WK;  // trip count, uniform over the workgroup
-  const int tile16_0 = (blockIdx.x * kWavesN + wave_n) * T;
+  const int tile16_0 = (blockIdx.x * kWavesN + wave_n) * TC;
   const int m_base = blockIdx.z * (16 * MT);
   uint8_t *const xlds = lds + kg * (2 * kStageBytes);
 
@@ -164,10 +172,11 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   uint32_t szlane[T];  // byte offset of this lane's column inside one [N] row of (scale, zero) pairs
 #pragma unroll
   for (int t = 0; t < T; ++t) {
-    int nt8 = 2 * (tile16_0 + t) + (c >> 3);
+    const int tcol = tile16_0 + (GATE ? 0 : t);
+    int nt8 = 2 * tcol + (c >> 3);
     nt8 = nt8 < n_tiles8 ? nt8 : n_tiles8 - 1;
     wlane[t] = static_cast<uint32_t>((static_cast<size_t>(nt8) * KT * 32 + ((c & 7) * 4 + b)) * Geo::WORDS * 4);
-    int ncol = 16 * (tile16_0 + t) + c;
+    int ncol = 16 * tcol + c;
     ncol = ncol < N ? ncol : N - 1;
     szlane[t] = static_cast<uint32_t>(ncol) * 4u;
   }
@@ -175,6 +184,8 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   // so a load costs no vector ALU work at all.  Every tensor is smaller than 4 GB (checked on the host).
   const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(wp, static_cast<uint32_t>(static_cast<size_t>(N) * K / 2));
   const __amdgpu_buffer_rsrc_t sz_rsrc = make_rsrc(sz, static_cast<uint32_t>(static_cast<size_t>(K / G) * N * 4));
+  const __amdgpu_buffer_rsrc_t w2_rsrc = make_rsrc(GATE ? wp2 : wp, static_cast<uint32_t>(static_cast<size_t>(N) * K / 2));
+  const __amdgpu_buffer_rsrc_t sz2_rsrc = make_rsrc(GATE ? sz2 : sz, static_cast<uint32_t>(static_cast<size_t>(K / G) * N * 4));
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
 
   auto load_weights = [&](wregs_t &r, int ci) {
@@ -182,24 +193,26 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     const uint32_t szchunk = static_cast<uint32_t>(ci) * Geo::NGRP * N * 4;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
+      const __amdgpu_buffer_rsrc_t wr = (GATE && t == 1) ? w2_rsrc : w_rsrc;
+      const __amdgpu_buffer_rsrc_t sr = (GATE && t == 1) ? sz2_rsrc : sz_rsrc;
 #pragma unroll
       for (int blk = 0; blk < Geo::NBLK; ++blk) {
         const uint32_t so = wchunk + blk * (32 * Geo::WORDS * 4);
         if constexpr (Geo::WORDS == 4) {
-          const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[t], so, kWeightCachePolicy);
+          const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(wr, wlane[t], so, kWeightCachePolicy);
 #pragma unroll
           for (int p = 0; p < 4; ++p) r.w[t][blk * 4 + p] = v[p];
         } else if constexpr (Geo::WORDS == 2) {
-          const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(w_rsrc, wlane[t], so, kWeightCachePolicy);
+          const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(wr, wlane[t], so, kWeightCachePolicy);
           r.w[t][blk * 2] = v[0];
           r.w[t][blk * 2 + 1] = v[1];
         } else {
-          r.w[t][blk] = __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, wlane[t], so, kWeightCachePolicy);
+          r.w[t][blk] = __builtin_amdgcn_raw_buffer_load_b32(wr, wlane[t], so, kWeightCachePolicy);
         }
       }
 #pragma unroll
       for (int g = 0; g < Geo::NGRP; ++g)
-        r.sz[t][g] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, szlane[t], szchunk + g * N * 4, 0);
+        r.sz[t][g] = __builtin_amdgcn_raw_buffer_load_b32(sr, szlane[t], szchunk + g * N * 4, 0);
     }
   };
 
@@ -327,31 +340,13 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
         const int i = base + j;
         const int phase = i / CPP;
         const uint32_t live = i < nloc ? 0xFFFFFFFFu : 0u;
-#ifndef E2H_DBG_NO_X
         if (j % CPP == 0) load_x(xstage[(j / CPP) % XD], phase + XD);
-#endif
         load_weights(ring[(j + PD) % NB], chunk_at(i + PD));
-#ifdef E2H_DBG_NO_COMPUTE
-        {
-          uint32_t h = 0;
-#pragma unroll
-          for (int t = 0; t < T; ++t) {
-#pragma unroll
-            for (int s2 = 0; s2 < Geo::STEPS; ++s2) h ^= ring[j % NB].w[t][s2];
-#pragma unroll
-            for (int g2 = 0; g2 < Geo::NGRP; ++g2) h ^= ring[j % NB].sz[t][g2];
-          }
-          acc[0][0][0] += __builtin_bit_cast(float, h & live & 0x3FFFFFFFu);
-        }
-#else
         compute_chunk(ring[j % NB], phase, j % CPP, live);
-#endif
-#ifndef E2H_DBG_NO_X
         if (j % CPP == CPP - 1) {
           store_x(xstage[(j / CPP + 1) % XD], phase + 1);
           lds_barrier();
         }
-#endif
       }
     }
   }
@@ -427,6 +422,19 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     }
   }
   if (kg != 0) return;
+  if constexpr (GATE) {
+    const int n = 16 * tile16_0 + c;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = m_base + 16 * mt + 4 * b + q;
+        const float gate = bf16_round(acc[0][mt][q]), up = bf16_round(acc[1][mt][q]);
+        const float act = bf16_round(gate / (1.0f + expf(-gate)));
+        if (n < N && m < M) y[static_cast<size_t>(m) * N + n] = f32_to_bf16_rne(act * up);
+      }
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const int n = 16 * (tile16_0 + t) + c;
@@ -444,6 +452,8 @@ struct LaunchArgs {
   const uint16_t *x;
   const int32_t *packed;
   const uint16_t *sz;
+  const int32_t *packed2;  // second weight matrix of the gated form, else null
+  const uint16_t *sz2;
   uint16_t *y;
   float *ws_partial;
   unsigned *ws_ticket;
@@ -451,12 +461,14 @@ struct LaunchArgs {
   hipStream_t stream;
 };
 
-template <int G, int IKT, int MT, int T, int WN, int WK>
+template <int G, int IKT, int MT, int T, int WN, int WK, bool GATE = false>
 int launch(const LaunchArgs &a) {
   const int tiles16 = (a.N + 15) / 16;
-  dim3 grid((tiles16 + WN * T - 1) / (WN * T), a.S, (a.M + 16 * MT - 1) / (16 * MT));
-  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
-                     reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz), a.y,
+  constexpr int TC = GATE ? 1 : T;
+  dim3 grid((tiles16 + WN * TC - 1) / (WN * TC), a.S, (a.M + 16 * MT - 1) / (16 * MT));
+  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK, GATE>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
+                     reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz),
+                     reinterpret_cast<const uint32_t *>(a.packed2), reinterpret_cast<const uint32_t *>(a.sz2), a.y,
                      a.ws_partial, a.ws_ticket, a.M, a.N, a.K);
   return launch_status();
 }
@@ -466,7 +478,7 @@ struct Shape {
   int t, wn, wk;
 };
 constexpr Shape kShapes[] = {{1, 4, 1}, {1, 4, 2}, {1, 4, 4}, {1, 3, 4}, {1, 2, 4}, {1, 2, 2}, {1, 1, 4},
-                             {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {2, 3, 2}, {4, 4, 1}};
+                             {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {2, 3, 2}, {4, 4, 1}, {1, 8, 1}};
 
 template <int G, int IKT>
 int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
@@ -477,7 +489,7 @@ int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
     if (mt == 2) return launch<G, IKT, 2, TV, WNV, WKV>(a);                     \
   }
     E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 4, 4) E2H_CASE(1, 3, 4) E2H_CASE(1, 2, 4) E2H_CASE(1, 2, 2)
-    E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1)
+    E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1) E2H_CASE(1, 8, 1)
 #undef E2H_CASE
     if (sh.t == 4) return launch<G, IKT, 4, 4, 4, 1>(a);
     if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1>(a);
@@ -527,6 +539,7 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
   LaunchArgs a;
   a.x = x; a.packed = packed; a.sz = scales_and_zeros; a.y = y;
+  a.packed2 = nullptr; a.sz2 = nullptr;
   a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
   a.stream = static_cast<hipStream_t>(stream);
   int mt = a.M <= 16 ? 1 : (a.M <= 32 ? 2 : 4);
@@ -598,4 +611,59 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     if (rc != E2H_OK) return rc;
   }
   return E2H_OK;
+}
+
+namespace e2h {
+namespace {
+
+template <int G>
+int dispatch_gate(int mt, int wn, const LaunchArgs &a) {
+#define E2H_GATE_CASE(MTV, WNV) \
+  if (mt == MTV && wn == WNV) return launch<G, 8, MTV, 2, WNV, 2, true>(a);
+  E2H_GATE_CASE(1, 4) E2H_GATE_CASE(2, 4) E2H_GATE_CASE(1, 3) E2H_GATE_CASE(2, 3) E2H_GATE_CASE(1, 2) E2H_GATE_CASE(2, 2)
+#undef E2H_GATE_CASE
+  return E2H_ERR_BAD_SHAPE;
+}
+
+}  // namespace
+}  // namespace e2h
+
+extern "C" int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_gate, const uint16_t *sz_gate,
+                                     const int32_t *packed_up, const uint16_t *sz_up, uint16_t *y, int64_t m, int64_t n,
+                                     int64_t k, int groupsize, int inner_k_tiles, void *stream) {
+  using namespace e2h;
+  if (!x || !packed_gate || !sz_gate || !packed_up || !sz_up || !y) return E2H_ERR_NULL_POINTER;
+  if (groupsize != 32 && groupsize != 64 && groupsize != 128) return E2H_ERR_BAD_GROUPSIZE;
+  if (inner_k_tiles != 8) return E2H_ERR_BAD_INNER_K_TILES;
+  if (m < 1 || m > 32 || n < 8 || k < 1 || (n % 8) != 0 || n > INT32_MAX || k > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if (k % groupsize != 0) return E2H_ERR_BAD_GROUPSIZE;
+  if (k % 128 != 0) return E2H_ERR_BAD_INNER_K_TILES;
+  if (!aligned16(x) || !aligned16(packed_gate) || !aligned16(sz_gate) || !aligned16(packed_up) || !aligned16(sz_up) ||
+      (reinterpret_cast<uintptr_t>(y) & 1u))
+    return E2H_ERR_MISALIGNED;
+  if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
+  LaunchArgs a;
+  a.x = x; a.packed = packed_gate; a.sz = sz_gate; a.packed2 = packed_up; a.sz2 = sz_up; a.y = y;
+  a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
+  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr;
+  a.stream = static_cast<hipStream_t>(stream);
+  const int mt = a.M <= 16 ? 1 : 2;
+  // column waves per workgroup: the count that leaves the fewest idle CUs in the last round of workgroups
+  const int tiles16 = (a.N + 15) / 16;
+  int wn = options().int4_col_waves;
+  if (wn < 2 || wn > 4) {
+    wn = 4;
+    double best = -1.0;
+    for (int cand = 4; cand >= 2; --cand) {
+      const int wgs = (tiles16 + cand - 1) / cand;
+      const int rounds = (wgs + kCUs - 1) / kCUs;
+      const double fill = static_cast<double>(wgs) / (static_cast<double>(rounds) * kCUs);
+      if (fill > best + 0.05) { best = fill; wn = cand; }
+    }
+  }
+  switch (groupsize) {
+    case 32: return dispatch_gate<32>(mt, wn, a);
+    case 64: return dispatch_gate<64>(mt, wn, a);
+    default: return dispatch_gate<128>(mt, wn, a);
+  }
 }

@@ -16,7 +16,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from . import ops
-from .quantize import find_multiple
+from .quantize import WeightOnlyInt4Linear, find_multiple
 
 # When True (default) and the tensors are bf16 on the GPU, RMSNorm, SiLU*mul and -- for single-token steps with
 # a KV cache -- RoPE + cache write + attention run as this package's fused kernels instead of chains of stock ops.
@@ -191,7 +191,20 @@ class FeedForward(nn.Module):
         self.w3 = nn.Linear(config.dim, config.intermediate_size, bias=False)
         self.w2 = nn.Linear(config.intermediate_size, config.dim, bias=False)
 
+    def _gate_fusable(self, x: Tensor) -> bool:
+        w1, w3 = self.w1, self.w3
+        if not (FUSED_DECODE and isinstance(w1, WeightOnlyInt4Linear) and isinstance(w3, WeightOnlyInt4Linear)):
+            return False
+        if w1.padding or w3.padding or torch.compiler.is_compiling():
+            return False
+        return ops.int4_gate_supported(x, w1, w3)
+
     def forward(self, x: Tensor) -> Tensor:
+        if self._gate_fusable(x):
+            # silu(w1 x) * w3 x in one launch: both products share the activation stream
+            y = ops.int4_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales_and_zeros,
+                                      self.w3.weight, self.w3.scales_and_zeros, self.w1.groupsize)
+            return self.w2(y.reshape(*x.shape[:-1], y.shape[-1]))
         a, b = self.w1(x), self.w3(x)
         if _fusable(a) and a.numel() % 8 == 0:
             return self.w2(ops.silu_mul(a, b))

@@ -258,6 +258,40 @@ def _int4_mm_impl(x, packed, groupsize, scales_and_zeros):
     return y
 
 
+def int4_gate_supported(x, w_gate, w_up):
+    """True when (x, two WeightOnlyInt4Linear modules) fit e2h_int4_mm_silu_gate's contract."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 32):
+        return False
+    pg, pu = w_gate.weight, w_up.weight
+    if pg.shape != pu.shape or pg.dim() != 4 or pg.shape[3] != 4 or w_gate.groupsize != w_up.groupsize:
+        return False
+    return w_gate.groupsize in (32, 64, 128) and w_gate.scales_and_zeros.shape == w_up.scales_and_zeros.shape
+
+
+def int4_mm_silu_gate(x, packed_gate, sz_gate, packed_up, sz_up, groupsize):
+    """bf16(bf16(silu(int4_mm(x, gate))) * int4_mm(x, up)) in one launch; x bf16 [M <= 32, K]."""
+    _need_gpu(x, packed_gate, sz_gate, packed_up, sz_up)
+    if x.dtype != torch.bfloat16 or sz_gate.dtype != torch.bfloat16 or sz_up.dtype != torch.bfloat16:
+        raise TypeError("int4_mm_silu_gate: bfloat16 activations and scales_and_zeros expected")
+    assert x.dim() == 2
+    n, k, ikt = _packed_dims(packed_gate)
+    if _packed_dims(packed_up) != (n, k, ikt):
+        raise RuntimeError("int4_mm_silu_gate: the two packed weights differ in shape")
+    m = x.shape[0]
+    if x.shape[1] != k:
+        raise RuntimeError(f"int4_mm_silu_gate: x has K={x.shape[1]}, packed weights have K={k}")
+    for sz in (sz_gate, sz_up):
+        if tuple(sz.shape) != (k // groupsize, n, 2):
+            raise RuntimeError(f"int4_mm_silu_gate: scales_and_zeros must be [{k // groupsize}, {n}, 2], got {tuple(sz.shape)}")
+    x, packed_gate, sz_gate = x.contiguous(), packed_gate.contiguous(), sz_gate.contiguous()
+    packed_up, sz_up = packed_up.contiguous(), sz_up.contiguous()
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    rc = _lib_for(x).e2h_int4_mm_silu_gate(_ptr(x), _ptr(packed_gate), _ptr(sz_gate), _ptr(packed_up), _ptr(sz_up), _ptr(y),
+                                           m, n, k, groupsize, ikt, _stream(x))
+    _lib.check(rc, "e2h_int4_mm_silu_gate")
+    return y
+
+
 # ---------------------------------------------------------------------------------------------
 # torch.library registrations (operator boundary that replaces the two aten int4 ops and the
 # F.linear * scales pair of the reference)

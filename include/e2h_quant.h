@@ -127,6 +127,17 @@ int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales
                 int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *workspace,
                 int64_t workspace_bytes, void *stream);
 
+/* Gated feed-forward front half in one launch:  y = F.silu(w1(x)) * w3(x)  for two WeightOnlyInt4Linear
+ * modules of equal shape (FeedForward.forward, reference models/model.py:343-344, with linear_forward_int4
+ * :445-453 for each product).  Rounding points as the reference's bfloat16 tensors: each product is rounded
+ * to bfloat16, silu's result is rounded, the final product is rounded.
+ *   x [m, k] bf16, packed_gate / packed_up [n/8, k/128, 32, 4] int32, sz_gate / sz_up [k/g, n, 2] bf16
+ *   -> y [m, n] bf16.  1 <= m <= 32 (decode batches; larger m: call e2h_int4_mm twice and e2h_silu_mul),
+ *   inner_k_tiles == 8, g in {32,64,128}, k % 128 == 0, n % 8 == 0; 16-byte aligned inputs. */
+int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_gate, const uint16_t *sz_gate,
+                          const int32_t *packed_up, const uint16_t *sz_up, uint16_t *y, int64_t m, int64_t n,
+                          int64_t k, int groupsize, int inner_k_tiles, void *stream);
+
 /* Recommended size in bytes of the workspace accepted by the matmul entry points (no reference counterpart). */
 int64_t e2h_workspace_bytes(void);
 

@@ -231,3 +231,42 @@ def test_int8_module_and_on_the_fly_handler_with_hooks():
     assert qo.normwise_rel_err(bf16_to_np(y), y_ref) <= TOL
     with pytest.raises(TypeError):
         model(x.float().to(DEV))
+
+
+# ---- gated feed-forward front half: silu(w1 x) * w3 x in one launch (reference models/model.py:343-344) ----
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32])
+@pytest.mark.parametrize("n,k,g", [(48, 512, 128), (688, 1024, 64), (200, 256, 32), (11008, 4096, 128)])
+def test_int4_gate_matches_oracle_and_unfused_path(m, n, k, g):
+    if n * k > 1 << 22 and m not in (1, 32):
+        pytest.skip("large shape: first and last batch size only")
+    codes1, sz1, p1, s1 = _int4_case(n, k, g, 8, seed=n + m)
+    codes2, sz2, p2, s2 = _int4_case(n, k, g, 8, seed=n + m + 7)
+    x = randn_bf16((m, k), std=1.0, seed=m * 31 + g)
+    xd = x.to(DEV)
+    y = ops.int4_mm_silu_gate(xd, p1, s1, p2, s2, g)
+    assert y.dtype == torch.bfloat16 and y.shape == (m, n)
+    # float oracle of the unrounded expression
+    a = qo.int4_linear_fp32(bf16_to_np(x), codes1, sz1, g).astype(np.float64)
+    b = qo.int4_linear_fp32(bf16_to_np(x), codes2, sz2, g).astype(np.float64)
+    ref = a / (1.0 + np.exp(-a)) * b
+    # three bf16 roundings (2^-9 each) on top of the matmul gate
+    assert qo.normwise_rel_err(bf16_to_np(y), ref) <= TOL
+    # same accumulation order as the single-matrix kernel with one K slice: identical bits
+    _lib.set_option("int4_k_slices", 1)
+    try:
+        ya = ops.int4_mm_direct(xd, p1, g, s1)
+        yb = ops.int4_mm_direct(xd, p2, g, s2)
+    finally:
+        _lib.set_option("int4_k_slices", 0)
+    assert torch.equal(y, ops.silu_mul(ya, yb))
+
+
+def test_int4_gate_rejects_what_it_does_not_cover():
+    codes, sz, p, s = _int4_case(48, 512, 128, 8)
+    x = randn_bf16((33, 512), seed=3).to(DEV)
+    with pytest.raises(RuntimeError):
+        ops.int4_mm_silu_gate(x, p, s, p, s, 128)           # m > 32
+    _, _, p4, s4 = _int4_case(48, 512, 128, 4)
+    with pytest.raises(RuntimeError):
+        ops.int4_mm_silu_gate(x[:4], p4, s4, p4, s4, 128)   # inner_k_tiles != 8
