@@ -173,11 +173,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
   const size_t row = blockIdx.x;
   const uint16_t *xr = x + row * dim;
   constexpr int kMaxPieces = 4;  // dim <= 256 * 8 * 4 = 8192 values are kept in registers, longer rows are re-read
-  u32x4_t keep[kMaxPieces];
+  u32x4_t keep[kMaxPieces], keepw[kMaxPieces];
   float ss = 0.f;
   int np = 0;
   for (int i = threadIdx.x * 8; i < dim; i += 2048, ++np) {
     u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+    if (np < kMaxPieces) keepw[np] = *reinterpret_cast<const u32x4_t *>(w + i);  // in flight across the reduction
     if (delta) {
       const u32x4_t dr = *reinterpret_cast<const u32x4_t *>(delta + row * dim + i);
 #pragma unroll
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
   np = 0;
   for (int i = threadIdx.x * 8; i < dim; i += 2048, ++np) {
     const u32x4_t raw = np < kMaxPieces ? keep[np] : *reinterpret_cast<const u32x4_t *>(src + i);
-    const u32x4_t wr = *reinterpret_cast<const u32x4_t *>(w + i);
+    const u32x4_t wr = np < kMaxPieces ? keepw[np] : *reinterpret_cast<const u32x4_t *>(w + i);
     u32x4_t o;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

@@ -114,11 +114,28 @@ struct Tuning {
 // wp2 / sz2, the gate and up projections of a feed-forward block); the epilogue writes
 // bf16(bf16(silu(bf16(gate))) * bf16(up)), the rounding points of  F.silu(w1(x)) * w3(x)  on bfloat16 tensors
 // (reference models/model.py:343-344).  Both products share one activation stream.
-template <int G, int IKT, int MT, int T, int WN, int WK, bool GATE = false>
+//
+// ROPE (one new token per sequence, x row m = sequence m): the product is the fused q | k | v projection; the
+// epilogue rounds it to bfloat16, rotates the interleaved pairs of the q and k heads in float32 by the angle of
+// position input_pos[0] (reference models/model.py:400-412), and writes q to q_out [B, H, D] and k, v straight
+// into the caches [B, Hkv, S, D] at that position (KVCache.update, reference models/model.py:94-104).
+enum Epilogue { kPlain = 0, kGate = 1, kRope = 2 };
+
+struct RopeArgs {
+  const uint16_t *freqs;     // [>= S, D/2, 2] bf16 (cos, sin)
+  uint16_t *q_out, *kc, *vc;
+  const int64_t *input_pos;  // [1] on the device
+  int H, Hkv, S, D;
+};
+
+template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain>
 __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
     const uint32_t *__restrict__ wp2, const uint32_t *__restrict__ sz2,
-    uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K) {
+    uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K,
+    RopeArgs rope) {
+  constexpr bool GATE = EPI == kGate;
+  static_assert(EPI != kRope || T == 1, "the rotary epilogue handles one column tile per wave");
   static_assert(!GATE || T == 2, "gate mode pairs exactly two weight matrices");
   constexpr int TC = GATE ? 1 : T;  // distinct column tiles per wave
   typedef Int4Geom<G, IKT> Geo;
@@ -325,11 +342,24 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   // loads hit cache, the arithmetic is neutralised with live = 0), and the trip count is rounded up to U.
   wregs_t ring[NB];
   u32x4_t xstage[XD][kPiecesPerThread];
+  int rope_pos = -1;
+  float rope_cs = 1.f, rope_sn = 0.f;
   if (C1 > C0) {
 #pragma unroll
     for (int d = 0; d < XD; ++d) load_x(xstage[d], d);
 #pragma unroll
     for (int i = 0; i < PD; ++i) load_weights(ring[i], chunk_at(i));
+    if constexpr (EPI == kRope) {
+      // the rotation's cos / sin depend on a position read from memory: fetch both now, behind the first
+      // weight loads, instead of as two dependent round trips at the very end
+      rope_pos = static_cast<int>(rope.input_pos[0]);
+      const int ncol = 16 * tile16_0 + c;
+      if (ncol < N && rope_pos >= 0 && rope_pos < rope.S && ncol < (rope.H + rope.Hkv) * rope.D) {
+        const uint32_t f = reinterpret_cast<const uint32_t *>(rope.freqs)[static_cast<size_t>(rope_pos) * (rope.D / 2) + ((ncol % rope.D) >> 1)];
+        rope_cs = __builtin_bit_cast(float, f << 16);
+        rope_sn = __builtin_bit_cast(float, f & 0xFFFF0000u);
+      }
+    }
     store_x(xstage[0], 0);
     lds_barrier();
     // invariant at the top of phase ph: LDS stage (ph & 1) holds the activations of phase ph, register set
@@ -422,6 +452,37 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     }
   }
   if (kg != 0) return;
+  if constexpr (EPI == kRope) {
+    const int n = 16 * tile16_0 + c;
+    const int D = rope.D, H = rope.H, Hkv = rope.Hkv;
+    const int head = n / D, d = n % D;
+    const int pos = rope_pos;
+    const bool in_range = n < N && pos >= 0 && pos < rope.S;
+    const bool rotated = head < H + Hkv;
+    const float cs = rope_cs, sn = rope_sn;
+    uint16_t *dst;  // element (m = 0) of this lane's column; rows are row_stride apart
+    size_t row_stride;
+    if (head < H) {
+      dst = rope.q_out + static_cast<size_t>(head) * D + d;
+      row_stride = static_cast<size_t>(H) * D;
+    } else {
+      const int hk = rotated ? head - H : head - H - Hkv;
+      dst = (rotated ? rope.kc : rope.vc) + (static_cast<size_t>(hk) * rope.S + pos) * D + d;
+      row_stride = static_cast<size_t>(Hkv) * rope.S * D;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = m_base + 16 * mt + 4 * b + q;
+        const float own = bf16_round(acc[0][mt][q]);
+        const float other = __shfl_xor(own, 1);  // the pair's other column lives in the neighbouring lane
+        // even column: x0 * cos - x1 * sin; odd column: x1 * cos + x0 * sin (two rounded products, then the sum)
+        const float r = (c & 1) ? own * cs + other * sn : own * cs - other * sn;
+        if (in_range && m < M) dst[static_cast<size_t>(m) * row_stride] = f32_to_bf16_rne(rotated ? r : own);
+      }
+    return;
+  }
   if constexpr (GATE) {
     const int n = 16 * tile16_0 + c;
 #pragma unroll
@@ -455,21 +516,22 @@ struct LaunchArgs {
   const int32_t *packed2;  // second weight matrix of the gated form, else null
   const uint16_t *sz2;
   uint16_t *y;
+  RopeArgs rope;
   float *ws_partial;
   unsigned *ws_ticket;
   int M, N, K, S;
   hipStream_t stream;
 };
 
-template <int G, int IKT, int MT, int T, int WN, int WK, bool GATE = false>
+template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain>
 int launch(const LaunchArgs &a) {
   const int tiles16 = (a.N + 15) / 16;
-  constexpr int TC = GATE ? 1 : T;
+  constexpr int TC = EPI == kGate ? 1 : T;
   dim3 grid((tiles16 + WN * TC - 1) / (WN * TC), a.S, (a.M + 16 * MT - 1) / (16 * MT));
-  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK, GATE>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
+  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK, EPI>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
                      reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz),
                      reinterpret_cast<const uint32_t *>(a.packed2), reinterpret_cast<const uint32_t *>(a.sz2), a.y,
-                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K);
+                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K, a.rope);
   return launch_status();
 }
 
@@ -539,7 +601,7 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
   LaunchArgs a;
   a.x = x; a.packed = packed; a.sz = scales_and_zeros; a.y = y;
-  a.packed2 = nullptr; a.sz2 = nullptr;
+  a.packed2 = nullptr; a.sz2 = nullptr; a.rope = RopeArgs{};
   a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
   a.stream = static_cast<hipStream_t>(stream);
   int mt = a.M <= 16 ? 1 : (a.M <= 32 ? 2 : 4);
@@ -619,7 +681,7 @@ namespace {
 template <int G>
 int dispatch_gate(int mt, int wn, const LaunchArgs &a) {
 #define E2H_GATE_CASE(MTV, WNV) \
-  if (mt == MTV && wn == WNV) return launch<G, 8, MTV, 2, WNV, 2, true>(a);
+  if (mt == MTV && wn == WNV) return launch<G, 8, MTV, 2, WNV, 2, kGate>(a);
   E2H_GATE_CASE(1, 4) E2H_GATE_CASE(2, 4) E2H_GATE_CASE(1, 3) E2H_GATE_CASE(2, 3) E2H_GATE_CASE(1, 2) E2H_GATE_CASE(2, 2)
 #undef E2H_GATE_CASE
   return E2H_ERR_BAD_SHAPE;
@@ -645,7 +707,7 @@ extern "C" int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_ga
   LaunchArgs a;
   a.x = x; a.packed = packed_gate; a.sz = sz_gate; a.packed2 = packed_up; a.sz2 = sz_up; a.y = y;
   a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
-  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr;
+  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr; a.rope = RopeArgs{};
   a.stream = static_cast<hipStream_t>(stream);
   const int mt = a.M <= 16 ? 1 : 2;
   // column waves per workgroup: the count that leaves the fewest idle CUs in the last round of workgroups
@@ -665,5 +727,40 @@ extern "C" int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_ga
     case 32: return dispatch_gate<32>(mt, wn, a);
     case 64: return dispatch_gate<64>(mt, wn, a);
     default: return dispatch_gate<128>(mt, wn, a);
+  }
+}
+
+extern "C" int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
+                                   const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache,
+                                   const int64_t *input_pos, int64_t batch, int64_t n_head, int64_t n_kv_head,
+                                   int64_t head_dim, int64_t cache_len, int64_t k, int groupsize, int inner_k_tiles,
+                                   void *stream) {
+  using namespace e2h;
+  if (!x || !packed || !scales_and_zeros || !freqs_cis || !q_out || !k_cache || !v_cache || !input_pos) return E2H_ERR_NULL_POINTER;
+  if (groupsize != 32 && groupsize != 64 && groupsize != 128) return E2H_ERR_BAD_GROUPSIZE;
+  if (inner_k_tiles != 8) return E2H_ERR_BAD_INNER_K_TILES;
+  if (batch < 1 || batch > 32 || n_head < 1 || n_kv_head < 1 || head_dim < 2 || (head_dim % 2) != 0 || cache_len < 1 || k < 1)
+    return E2H_ERR_BAD_SHAPE;
+  const int64_t n = (n_head + 2 * n_kv_head) * head_dim;
+  if ((n % 8) != 0 || n > INT32_MAX || k > INT32_MAX || cache_len > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if (k % groupsize != 0) return E2H_ERR_BAD_GROUPSIZE;
+  if (k % 128 != 0) return E2H_ERR_BAD_INNER_K_TILES;
+  if (!aligned16(x) || !aligned16(packed) || !aligned16(scales_and_zeros) || (reinterpret_cast<uintptr_t>(freqs_cis) & 3u) ||
+      (reinterpret_cast<uintptr_t>(q_out) & 1u) || (reinterpret_cast<uintptr_t>(k_cache) & 1u) || (reinterpret_cast<uintptr_t>(v_cache) & 1u) ||
+      (reinterpret_cast<uintptr_t>(input_pos) & 7u))
+    return E2H_ERR_MISALIGNED;
+  if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
+  LaunchArgs a;
+  a.x = x; a.packed = packed; a.sz = scales_and_zeros; a.packed2 = nullptr; a.sz2 = nullptr; a.y = nullptr;
+  a.rope = RopeArgs{freqs_cis, q_out, k_cache, v_cache, input_pos, static_cast<int>(n_head), static_cast<int>(n_kv_head),
+                    static_cast<int>(cache_len), static_cast<int>(head_dim)};
+  a.M = static_cast<int>(batch); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
+  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr;
+  a.stream = static_cast<hipStream_t>(stream);
+  const bool two = a.M > 16;
+  switch (groupsize) {
+    case 32: return two ? launch<32, 8, 2, 1, 4, 2, kRope>(a) : launch<32, 8, 1, 1, 4, 2, kRope>(a);
+    case 64: return two ? launch<64, 8, 2, 1, 4, 2, kRope>(a) : launch<64, 8, 1, 1, 4, 2, kRope>(a);
+    default: return two ? launch<128, 8, 2, 1, 4, 2, kRope>(a) : launch<128, 8, 1, 1, 4, 2, kRope>(a);
   }
 }

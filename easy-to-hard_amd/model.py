@@ -21,6 +21,9 @@ from .quantize import WeightOnlyInt4Linear, find_multiple
 # When True (default) and the tensors are bf16 on the GPU, RMSNorm, SiLU*mul and -- for single-token steps with
 # a KV cache -- RoPE + cache write + attention run as this package's fused kernels instead of chains of stock ops.
 FUSED_DECODE = True
+# finer switches under FUSED_DECODE (both on by default; tests and measurements turn them off to compare)
+FUSE_GATE = True            # silu(w1 x) * w3 x as one int4 launch
+FUSE_ROPE_PROJECTION = True  # q|k|v projection + RoPE + cache write as one int4 launch
 
 
 def _fusable(t: Tensor) -> bool:
@@ -161,9 +164,16 @@ class Attention(nn.Module):
         kv_size = self.n_local_heads * self.head_dim
         if self.can_fuse_decode(x, fully_causal):
             # one new token per sequence: RoPE + cache write in one kernel, then attention over the live positions only
-            qkv = self.wqkv(x).view(bsz, -1)
-            q = ops.rope_kv_write(qkv, self.freqs_table, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos,
-                                  self.n_head, self.n_local_heads, self.head_dim)
+            w = self.wqkv
+            if FUSE_ROPE_PROJECTION and isinstance(w, WeightOnlyInt4Linear) and ops.int4_rope_kv_supported(x, w, self.freqs_table, self.kv_cache.k_cache):
+                # projection, rotation and cache write in one launch
+                q = ops.int4_mm_rope_kv(x.view(bsz, -1), w.weight, w.scales_and_zeros, w.groupsize, self.freqs_table,
+                                        self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, self.n_head,
+                                        self.n_local_heads, self.head_dim)
+            else:
+                qkv = w(x).view(bsz, -1)
+                q = ops.rope_kv_write(qkv, self.freqs_table, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos,
+                                      self.n_head, self.n_local_heads, self.head_dim)
             y = ops.decode_attention(q, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, self.left_pad_mask_pos)
             return self.wo(y.view(bsz, 1, self.dim))
         q, k, v = self.wqkv(x).split([self.dim, kv_size, kv_size], dim=-1)
@@ -193,7 +203,7 @@ class FeedForward(nn.Module):
 
     def _gate_fusable(self, x: Tensor) -> bool:
         w1, w3 = self.w1, self.w3
-        if not (FUSED_DECODE and isinstance(w1, WeightOnlyInt4Linear) and isinstance(w3, WeightOnlyInt4Linear)):
+        if not (FUSED_DECODE and FUSE_GATE and isinstance(w1, WeightOnlyInt4Linear) and isinstance(w3, WeightOnlyInt4Linear)):
             return False
         if w1.padding or w3.padding or torch.compiler.is_compiling():
             return False

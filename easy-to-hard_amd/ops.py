@@ -398,6 +398,42 @@ def rope_kv_write(qkv, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head
     return q
 
 
+def int4_rope_kv_supported(x, wqkv, freqs_cis, k_cache):
+    """True when the fused projection + RoPE + cache write covers (x [B, 1, K], a WeightOnlyInt4Linear)."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 32):
+        return False
+    p = wqkv.weight
+    if p.dim() != 4 or p.shape[3] != 4 or wqkv.groupsize not in (32, 64, 128) or wqkv.padding:
+        return False
+    return freqs_cis.shape[0] >= k_cache.shape[2]
+
+
+def int4_mm_rope_kv(x, packed, scales_and_zeros, groupsize, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head, head_dim):
+    """x bf16 [B <= 32, K] (one new token per sequence) times the tile-packed fused q|k|v weight, then RoPE and
+    the cache write of rope_kv_write, in one launch.  Returns the rotated q [B, H, D]."""
+    _need_gpu(x, packed, scales_and_zeros, freqs_cis, k_cache, v_cache, input_pos)
+    assert x.dtype == torch.bfloat16 and scales_and_zeros.dtype == torch.bfloat16 and freqs_cis.dtype == torch.bfloat16
+    assert input_pos.dtype == torch.int64 and input_pos.numel() >= 1 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and freqs_cis.is_contiguous() and x.dim() == 2
+    n, k, ikt = _packed_dims(packed)
+    bsz = x.shape[0]
+    if n != (n_head + 2 * n_kv_head) * head_dim or x.shape[1] != k:
+        raise RuntimeError(f"int4_mm_rope_kv: weight is [{n}, {k}], expected [{(n_head + 2 * n_kv_head) * head_dim}, {x.shape[1]}]")
+    if tuple(scales_and_zeros.shape) != (k // groupsize, n, 2):
+        raise RuntimeError(f"int4_mm_rope_kv: scales_and_zeros must be [{k // groupsize}, {n}, 2], got {tuple(scales_and_zeros.shape)}")
+    if k_cache.shape[0] < bsz or k_cache.shape[1] != n_kv_head or k_cache.shape[3] != head_dim or v_cache.shape != k_cache.shape:
+        raise RuntimeError("int4_mm_rope_kv: caches must be [>= B, Hkv, S, D]")
+    if freqs_cis.shape[0] < k_cache.shape[2] or tuple(freqs_cis.shape[1:]) != (head_dim // 2, 2):
+        raise RuntimeError("int4_mm_rope_kv: freqs_cis must be [>= S, D/2, 2]")
+    x, packed, sz = x.contiguous(), packed.contiguous(), scales_and_zeros.contiguous()
+    q = torch.empty((bsz, n_head, head_dim), dtype=torch.bfloat16, device=x.device)
+    rc = _lib_for(x).e2h_int4_mm_rope_kv(_ptr(x), _ptr(packed), _ptr(sz), _ptr(freqs_cis), _ptr(q), _ptr(k_cache), _ptr(v_cache),
+                                         _ptr(input_pos), bsz, n_head, n_kv_head, head_dim, k_cache.shape[2], k, groupsize, ikt,
+                                         _stream(x))
+    _lib.check(rc, "e2h_int4_mm_rope_kv")
+    return q
+
+
 def decode_attention(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, scale=None):
     """q bf16 [B, H, D] against caches [Bmax, Hkv, S, D] up to and including input_pos -> bf16 [B, H, D]."""
     _need_gpu(q, k_cache, v_cache, input_pos)

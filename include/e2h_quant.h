@@ -138,6 +138,23 @@ int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_gate, const u
                           const int32_t *packed_up, const uint16_t *sz_up, uint16_t *y, int64_t m, int64_t n,
                           int64_t k, int groupsize, int inner_k_tiles, void *stream);
 
+/* Decode-step attention front half in one launch: the fused q|k|v projection of a WeightOnlyInt4Linear
+ * (Attention.forward, reference models/model.py:283-296: wqkv, split, apply_rotary_emb on q and k :400-412,
+ * KVCache.update :94-104) for ONE new token per sequence.  Row b of x is sequence b.
+ *   x [batch, k] bf16, packed [n/8, k/128, 32, 4] int32 with n = (n_head + 2*n_kv_head) * head_dim,
+ *   scales_and_zeros [k/g, n, 2] bf16, freqs_cis [>= cache_len, head_dim/2, 2] bf16 (cos, sin),
+ *   input_pos [1] int64 on the device (the position being written; a position outside [0, cache_len)
+ *   writes nothing).
+ *   -> q_out [batch, n_head, head_dim] bf16 (rotated), k_cache / v_cache [batch, n_kv_head, cache_len,
+ *   head_dim] bf16 updated at input_pos (k rotated).  The projection is rounded to bfloat16 before the
+ *   rotation, which is evaluated in float32 and rounded again, as in the reference.
+ * 1 <= batch <= 32, inner_k_tiles == 8, g in {32,64,128}, k % 128 == 0, n % 8 == 0, head_dim even. */
+int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
+                        const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache,
+                        const int64_t *input_pos, int64_t batch, int64_t n_head, int64_t n_kv_head,
+                        int64_t head_dim, int64_t cache_len, int64_t k, int groupsize, int inner_k_tiles,
+                        void *stream);
+
 /* Recommended size in bytes of the workspace accepted by the matmul entry points (no reference counterpart). */
 int64_t e2h_workspace_bytes(void);
 

@@ -270,3 +270,67 @@ def test_int4_gate_rejects_what_it_does_not_cover():
     _, _, p4, s4 = _int4_case(48, 512, 128, 4)
     with pytest.raises(RuntimeError):
         ops.int4_mm_silu_gate(x[:4], p4, s4, p4, s4, 128)   # inner_k_tiles != 8
+
+
+# ---- fused q|k|v projection + RoPE + KV-cache write (reference models/model.py:283-296, :400-412, :94-104) ----
+
+@pytest.mark.parametrize("bsz", [1, 3, 16, 32])
+@pytest.mark.parametrize("n_head,n_kv,d,k,g", [(4, 4, 64, 256, 32), (8, 2, 64, 512, 64), (32, 32, 128, 4096, 128), (6, 3, 128, 384, 128)])
+def test_int4_rope_kv_matches_two_kernel_path_and_stock_ops(bsz, n_head, n_kv, d, k, g):
+    from easy_to_hard_amd.model import apply_rotary_emb, precompute_freqs_cis
+
+    if k == 4096 and bsz not in (1, 32):
+        pytest.skip("large shape: first and last batch size only")
+    n = (n_head + 2 * n_kv) * d
+    s_max, pos = 80, 37
+    codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=n + bsz)
+    x = randn_bf16((bsz, k), std=1.0, seed=bsz * 17 + g).to(DEV)
+    gen = torch.Generator().manual_seed(n_head + d)
+    kc0 = torch.randn((bsz + 1, n_kv, s_max, d), generator=gen).to(torch.bfloat16).to(DEV)
+    vc0 = torch.randn((bsz + 1, n_kv, s_max, d), generator=gen).to(torch.bfloat16).to(DEV)
+    freqs = precompute_freqs_cis(s_max, d, 10000, device=DEV)
+    input_pos = torch.tensor([pos], device=DEV)
+
+    kc, vc = kc0.clone(), vc0.clone()
+    q = ops.int4_mm_rope_kv(x, packed_d, sz_d, g, freqs, kc, vc, input_pos, n_head, n_kv, d)
+
+    # two-kernel path with the same accumulation order (one K slice): identical bits
+    _lib.set_option("int4_k_slices", 1)
+    try:
+        qkv = ops.int4_mm_direct(x, packed_d, g, sz_d)
+    finally:
+        _lib.set_option("int4_k_slices", 0)
+    kc2, vc2 = kc0.clone(), vc0.clone()
+    q2 = ops.rope_kv_write(qkv, freqs, kc2, vc2, input_pos, n_head, n_kv, d)
+    assert torch.equal(q, q2) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    # only position `pos` of the first bsz sequences changed
+    untouched = torch.ones(s_max, dtype=torch.bool, device=DEV)
+    untouched[pos] = False
+    assert torch.equal(kc[:, :, untouched], kc0[:, :, untouched]) and torch.equal(kc[bsz], kc0[bsz])
+    assert torch.equal(vc[:, :, untouched], vc0[:, :, untouched]) and torch.equal(vc[bsz], vc0[bsz])
+
+    # stock ops on the oracle's projection (float32 oracle rounded to bf16 may differ from the kernel's in the last
+    # bit, so the comparison is by tolerance)
+    y_ref = torch.from_numpy(qo.int4_linear_fp32(bf16_to_np(x.cpu()), codes, sz, g)).to(torch.bfloat16).to(DEV)
+    qr, kr, vr = y_ref.view(bsz, 1, -1).split([n_head * d, n_kv * d, n_kv * d], dim=-1)
+    fc = freqs[input_pos]
+    q_ref = apply_rotary_emb(qr.view(bsz, 1, n_head, d), fc).squeeze(1)
+    k_ref = apply_rotary_emb(kr.view(bsz, 1, n_kv, d), fc).squeeze(1)
+    scale = float(y_ref.float().abs().max())
+    assert (q.float() - q_ref.float()).abs().max() <= TOL * scale
+    assert (kc[:bsz, :, pos].float() - k_ref.float()).abs().max() <= TOL * scale
+    assert (vc[:bsz, :, pos].float() - vr.view(bsz, n_kv, d).float()).abs().max() <= TOL * scale
+
+
+def test_int4_rope_kv_ignores_out_of_range_position():
+    n_head, n_kv, d, k, g, bsz, s_max = 4, 4, 64, 256, 32, 2, 16
+    _, _, packed_d, sz_d = _int4_case((n_head + 2 * n_kv) * d, k, g, 8)
+    from easy_to_hard_amd.model import precompute_freqs_cis
+
+    x = randn_bf16((bsz, k), seed=1).to(DEV)
+    kc0 = torch.zeros((bsz, n_kv, s_max, d), dtype=torch.bfloat16, device=DEV)
+    kc, vc = kc0.clone(), kc0.clone()
+    freqs = precompute_freqs_cis(s_max, d, 10000, device=DEV)
+    ops.int4_mm_rope_kv(x, packed_d, sz_d, g, freqs, kc, vc, torch.tensor([s_max], device=DEV), n_head, n_kv, d)
+    torch.cuda.synchronize()
+    assert torch.equal(kc, kc0) and torch.equal(vc, kc0)
