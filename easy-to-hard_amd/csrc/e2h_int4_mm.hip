@@ -174,8 +174,9 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   const int S = gridDim.y;
   const int ks = blockIdx.y;
   // workgroup slice [C0, C1) of the chunks, then this k-group's part [c0, c1) of it
-  const int C0 = static_cast<int>((static_cast<long long>(nchunks) * ks) / S);
-  const int C1 = static_cast<int>((static_cast<long long>(nchunks) * (ks + 1)) / S);
+  // (32-bit arithmetic: nchunks < 2^24 and S <= 64 on every path the host takes)
+  const int C0 = S == 1 ? 0 : static_cast<int>((static_cast<unsigned>(nchunks) * static_cast<unsigned>(ks)) / static_cast<unsigned>(S));
+  const int C1 = S == 1 ? nchunks : static_cast<int>((static_cast<unsigned>(nchunks) * static_cast<unsigned>(ks + 1)) / static_cast<unsigned>(S));
   const int c0 = C0 + ((C1 - C0) * kg) / WK;
   const int c1 = C0 + ((C1 - C0) * (kg + 1)) / WK;
   const int nloc = c1 - c0;
@@ -540,7 +541,7 @@ struct Shape {
   int t, wn, wk;
 };
 constexpr Shape kShapes[] = {{1, 4, 1}, {1, 4, 2}, {1, 4, 4}, {1, 3, 4}, {1, 2, 4}, {1, 2, 2}, {1, 1, 4},
-                             {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {2, 3, 2}, {4, 4, 1}, {1, 8, 1}};
+                             {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {2, 3, 2}, {4, 4, 1}};
 
 template <int G, int IKT>
 int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
@@ -551,7 +552,7 @@ int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
     if (mt == 2) return launch<G, IKT, 2, TV, WNV, WKV>(a);                     \
   }
     E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 4, 4) E2H_CASE(1, 3, 4) E2H_CASE(1, 2, 4) E2H_CASE(1, 2, 2)
-    E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1) E2H_CASE(1, 8, 1)
+    E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1)
 #undef E2H_CASE
     if (sh.t == 4) return launch<G, IKT, 4, 4, 4, 1>(a);
     if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1>(a);

@@ -133,3 +133,36 @@ def test_graph_replays_match_eager_every_time():
         torch.cuda.synchronize()
         assert torch.equal(eager, replay), i
         cur = eager
+
+
+@pytest.mark.parametrize("mode,g,label,expect", [("int8", 128, "", "modelint8.pth"), ("int4", 64, "_x_", "model_x_int4.g64.pth")])
+def test_quantize_writer_names_keys_and_reload(tmp_path, mode, g, label, expect):
+    """quantize() (reference models/quantize.py:669-754): output file name convention (:707, :718), state-dict keys
+    and dtypes of the two weight-only modes, and that the file loads into a converted model."""
+    ckpt_dir = tmp_path / "tiny-test"
+    ckpt_dir.mkdir()
+    model = _tiny()
+    torch.save(model.to(torch.bfloat16).state_dict(), ckpt_dir / "model.pth")
+    out = e2h.quantize(ckpt_dir / "model.pth", mode, g, label)
+    assert out == ckpt_dir / expect and out.is_file()
+    sd = torch.load(out, weights_only=True)
+    lin = "layers.0.attention.wqkv"
+    with torch.device("meta"):
+        rt = Transformer.from_name("tiny-test")
+    n, k = model.layers[0].attention.wqkv.weight.shape
+    if mode == "int8":
+        assert sd[lin + ".weight"].dtype == torch.int8 and sd[lin + ".scales"].dtype == torch.bfloat16
+        assert tuple(sd[lin + ".weight"].shape) == (n, k) and tuple(sd[lin + ".scales"].shape) == (n,)
+        e2h.WeightOnlyInt8QuantHandler(rt).convert_for_runtime()
+    else:
+        assert sd[lin + ".weight"].dtype == torch.int32 and tuple(sd[lin + ".weight"].shape) == (n // 8, k // 128, 32, 4)
+        assert sd[lin + ".scales_and_zeros"].dtype == torch.bfloat16 and tuple(sd[lin + ".scales_and_zeros"].shape) == (k // g, n, 2)
+        e2h.WeightOnlyInt4QuantHandler(rt, g).convert_for_runtime()
+    assert sd["tok_embeddings.weight"].dtype == torch.bfloat16  # non-linear entries pass through untouched
+    rt.load_state_dict(sd, assign=True)
+    rt = rt.to(device=DEV, dtype=torch.bfloat16).eval()
+    rt.setup_caches(2, 7)
+    ids = torch.randint(0, 512, (2, 7), generator=torch.Generator().manual_seed(3)).to(DEV)
+    with torch.no_grad():
+        logits = rt(ids, torch.arange(7, device=DEV))
+    assert logits.shape == (2, 7, 512) and torch.isfinite(logits.float()).all()
