@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0
 # `bench.py --gemv-only`, scaled by a 256 MiB copy; the summary with the commands is in
 # profiles/int4_skinny_mm_7b_decode_bs32.md.  Counters cannot be read from inside this process, so the figure is
 # recorded here for the configuration it was measured on and reported as null for any other.
-MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32): 29_440_000}
+MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32): 33_440_000}
 
 
 def parse_args():
