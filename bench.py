@@ -46,6 +46,11 @@ def parse_args():
     ap.add_argument("--max-new", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--gemv-reps", type=int, default=20)
+    ap.add_argument("--per-shape", default="",
+                    help="comma-separated row counts M: time every distinct quantized-linear shape of the model at each M "
+                         "(all layers' instances back to back, so the weights rotate) and print one JSON line")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="launch-geometry override passed to e2h_set_option (experiments)")
     ap.add_argument("--gemv-only", action="store_true",
                     help="only the back-to-back dequant-GEMV pass plus a 256 MiB calibration copy (for counter runs)")
     return ap.parse_args()
@@ -143,6 +148,52 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
     }
 
 
+def measure_per_shape(model, rows_list, reps=6):
+    """Average launch duration of each distinct quantized-linear shape, replayed from a HIP graph and timed with events on
+    the launch stream; the instances of a shape in different layers have different weights, so nothing stays cached."""
+    import torch
+
+    import easy_to_hard_amd as e2h
+
+    dev = torch.device("cuda", 0)
+    groups = {}
+    for name, mod in quantized_linears(model):
+        groups.setdefault((name.rpartition(".")[2], mod.out_features, mod.in_features), []).append(mod)
+    out = []
+    for (leaf, n, k), mods in groups.items():
+        for m in rows_list:
+            x = torch.randn((m, k), device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+            def one_pass():
+                for mod in mods:
+                    mod(x)
+
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):
+                one_pass()
+            torch.cuda.current_stream(dev).wait_stream(side)
+            graph = torch.cuda.CUDAGraph()  # replayed: host launch cost would otherwise hide the short kernels
+            with torch.cuda.graph(graph):
+                one_pass()
+            graph.replay()
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(reps):
+                graph.replay()
+            stop.record()
+            torch.cuda.synchronize()
+            del graph
+            us = start.elapsed_time(stop) * 1e3 / (reps * len(mods))
+            nbytes = algorithmic_bytes(mods[0], m)
+            int4 = isinstance(mods[0], e2h.WeightOnlyInt4Linear)
+            out.append({"linear": leaf, "n": n, "k": k, "m": m, "instances": len(mods), "us": round(us, 2),
+                        "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                        "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "kind": "int4" if int4 else "int8"})
+    return out
+
+
 def measure_cpu_baseline(model, batch, groupsize):
     """Reference CPU path on the host cores: one layer's five linears + the LM head, extrapolated."""
     import torch
@@ -206,6 +257,9 @@ def main():
     from easy_to_hard_amd.model import ModelArgs, random_quantized_transformer
 
     _lib.load()  # no fallback: fail here if the HIP library is not built
+    for item in args.option:
+        name, _, value = item.partition("=")
+        _lib.set_option(name, int(value))
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -216,6 +270,11 @@ def main():
     build_s = time.time() - t0
 
     batch, t_prompt = args.batch, args.prompt
+    if args.per_shape:
+        rows_list = [int(v) for v in args.per_shape.split(",") if v]
+        print(json.dumps({"per_shape": measure_per_shape(model, rows_list), "model": args.model, "mode": args.mode,
+                          "groupsize": args.groupsize if args.mode == "int4" else None}))
+        return
     if args.gemv_only:
         # counter-collection mode: the GEMV pass and a plain copy of known size (its FETCH_SIZE / WRITE_SIZE
         # readings calibrate the counters: 256 MiB read, 256 MiB written per copy)

@@ -314,9 +314,13 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
                    int64_t workspace_bytes, hipStream_t stream) {
   Args8 a;
   a.q = q; a.scales = scales; a.N = N; a.K = K; a.stream = stream;
-  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int m_chunks = (M + 16 * mt - 1) / (16 * mt);
   const int tiles16 = (N + 15) / 16;
+  // 33 ... 64 rows: the 64-row shape has no K split, so narrow matrices (fewer column blocks than CUs) run as
+  // two 32-row slabs with the K-split shapes instead (measured 2.5x ... 3x faster at N = 4096, slower at N >= 11008)
+  int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  if (M > 32 && M <= 64 && (tiles16 + 3) / 4 < kCUs8) mt = 2;
+  if (options().row_tiles) mt = options().row_tiles;
+  const int m_chunks = (M + 16 * mt - 1) / (16 * mt);
   const int nchunks = K / kChunk;
   const bool have_ws = workspace && workspace_bytes >= static_cast<int64_t>(kTicketBytes8) + (int64_t{1} << 20);
   int t = 1, wk = 2, s = 1;

@@ -260,7 +260,7 @@ def _int4_mm_impl(x, packed, groupsize, scales_and_zeros):
 
 def int4_gate_supported(x, w_gate, w_up):
     """True when (x, two WeightOnlyInt4Linear modules) fit e2h_int4_mm_silu_gate's contract."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 32):
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 64):
         return False
     pg, pu = w_gate.weight, w_up.weight
     if pg.shape != pu.shape or pg.dim() != 4 or pg.shape[3] != 4 or w_gate.groupsize != w_up.groupsize:
@@ -269,7 +269,7 @@ def int4_gate_supported(x, w_gate, w_up):
 
 
 def int4_mm_silu_gate(x, packed_gate, sz_gate, packed_up, sz_up, groupsize):
-    """bf16(bf16(silu(int4_mm(x, gate))) * int4_mm(x, up)) in one launch; x bf16 [M <= 32, K]."""
+    """bf16(bf16(silu(int4_mm(x, gate))) * int4_mm(x, up)) in one launch; x bf16 [M <= 64, K]."""
     _need_gpu(x, packed_gate, sz_gate, packed_up, sz_up)
     if x.dtype != torch.bfloat16 or sz_gate.dtype != torch.bfloat16 or sz_up.dtype != torch.bfloat16:
         raise TypeError("int4_mm_silu_gate: bfloat16 activations and scales_and_zeros expected")
@@ -400,7 +400,7 @@ def rope_kv_write(qkv, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head
 
 def int4_rope_kv_supported(x, wqkv, freqs_cis, k_cache):
     """True when the fused projection + RoPE + cache write covers (x [B, 1, K], a WeightOnlyInt4Linear)."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 32):
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 64):
         return False
     p = wqkv.weight
     if p.dim() != 4 or p.shape[3] != 4 or wqkv.groupsize not in (32, 64, 128) or wqkv.padding:
@@ -409,7 +409,7 @@ def int4_rope_kv_supported(x, wqkv, freqs_cis, k_cache):
 
 
 def int4_mm_rope_kv(x, packed, scales_and_zeros, groupsize, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head, head_dim):
-    """x bf16 [B <= 32, K] (one new token per sequence) times the tile-packed fused q|k|v weight, then RoPE and
+    """x bf16 [B <= 64, K] (one new token per sequence) times the tile-packed fused q|k|v weight, then RoPE and
     the cache write of rope_kv_write, in one launch.  Returns the rotated q [B, H, D]."""
     _need_gpu(x, packed, scales_and_zeros, freqs_cis, k_cache, v_cache, input_pos)
     assert x.dtype == torch.bfloat16 and scales_and_zeros.dtype == torch.bfloat16 and freqs_cis.dtype == torch.bfloat16

@@ -39,7 +39,7 @@ int e2h_abi_version(void);
 const char *e2h_status_string(int status);
 
 /* Tuning knobs for experiments: launch-geometry overrides such as "int4_rows_per_wave", "int4_k_slices", "int4_k_groups",
- * "int4_col_waves", "int8_rows_per_wave", "int8_k_groups", "int8_k_slices", "int8_force_generic";
+ * "int4_col_waves", "int8_rows_per_wave", "int8_k_groups", "int8_k_slices", "int8_force_generic", "row_tiles";
  * value 0 restores the built-in heuristic.  Not thread safe; set before launching. */
 int e2h_set_option(const char *name, int value);
 
@@ -132,7 +132,7 @@ int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales
  * :445-453 for each product).  Rounding points as the reference's bfloat16 tensors: each product is rounded
  * to bfloat16, silu's result is rounded, the final product is rounded.
  *   x [m, k] bf16, packed_gate / packed_up [n/8, k/128, 32, 4] int32, sz_gate / sz_up [k/g, n, 2] bf16
- *   -> y [m, n] bf16.  1 <= m <= 32 (decode batches; larger m: call e2h_int4_mm twice and e2h_silu_mul),
+ *   -> y [m, n] bf16.  1 <= m <= 64 (decode batches; larger m: call e2h_int4_mm twice and e2h_silu_mul),
  *   inner_k_tiles == 8, g in {32,64,128}, k % 128 == 0, n % 8 == 0; 16-byte aligned inputs. */
 int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_gate, const uint16_t *sz_gate,
                           const int32_t *packed_up, const uint16_t *sz_up, uint16_t *y, int64_t m, int64_t n,
@@ -148,7 +148,7 @@ int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_gate, const u
  *   -> q_out [batch, n_head, head_dim] bf16 (rotated), k_cache / v_cache [batch, n_kv_head, cache_len,
  *   head_dim] bf16 updated at input_pos (k rotated).  The projection is rounded to bfloat16 before the
  *   rotation, which is evaluated in float32 and rounded again, as in the reference.
- * 1 <= batch <= 32, inner_k_tiles == 8, g in {32,64,128}, k % 128 == 0, n % 8 == 0, head_dim even. */
+ * 1 <= batch <= 64, inner_k_tiles == 8, g in {32,64,128}, k % 128 == 0, n % 8 == 0, head_dim even. */
 int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
                         const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache,
                         const int64_t *input_pos, int64_t batch, int64_t n_head, int64_t n_kv_head,

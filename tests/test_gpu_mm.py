@@ -235,11 +235,11 @@ def test_int8_module_and_on_the_fly_handler_with_hooks():
 
 # ---- gated feed-forward front half: silu(w1 x) * w3 x in one launch (reference models/model.py:343-344) ----
 
-@pytest.mark.parametrize("m", [1, 5, 16, 17, 32])
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 33, 64])
 @pytest.mark.parametrize("n,k,g", [(48, 512, 128), (688, 1024, 64), (200, 256, 32), (11008, 4096, 128)])
 def test_int4_gate_matches_oracle_and_unfused_path(m, n, k, g):
-    if n * k > 1 << 22 and m not in (1, 32):
-        pytest.skip("large shape: first and last batch size only")
+    if n * k > 1 << 22 and m not in (1, 32, 64):
+        pytest.skip("large shape: three batch sizes only")
     codes1, sz1, p1, s1 = _int4_case(n, k, g, 8, seed=n + m)
     codes2, sz2, p2, s2 = _int4_case(n, k, g, 8, seed=n + m + 7)
     x = randn_bf16((m, k), std=1.0, seed=m * 31 + g)
@@ -264,9 +264,9 @@ def test_int4_gate_matches_oracle_and_unfused_path(m, n, k, g):
 
 def test_int4_gate_rejects_what_it_does_not_cover():
     codes, sz, p, s = _int4_case(48, 512, 128, 8)
-    x = randn_bf16((33, 512), seed=3).to(DEV)
+    x = randn_bf16((65, 512), seed=3).to(DEV)
     with pytest.raises(RuntimeError):
-        ops.int4_mm_silu_gate(x, p, s, p, s, 128)           # m > 32
+        ops.int4_mm_silu_gate(x, p, s, p, s, 128)           # m > 64
     _, _, p4, s4 = _int4_case(48, 512, 128, 4)
     with pytest.raises(RuntimeError):
         ops.int4_mm_silu_gate(x[:4], p4, s4, p4, s4, 128)   # inner_k_tiles != 8
@@ -274,13 +274,13 @@ def test_int4_gate_rejects_what_it_does_not_cover():
 
 # ---- fused q|k|v projection + RoPE + KV-cache write (reference models/model.py:283-296, :400-412, :94-104) ----
 
-@pytest.mark.parametrize("bsz", [1, 3, 16, 32])
+@pytest.mark.parametrize("bsz", [1, 3, 16, 32, 40, 64])
 @pytest.mark.parametrize("n_head,n_kv,d,k,g", [(4, 4, 64, 256, 32), (8, 2, 64, 512, 64), (32, 32, 128, 4096, 128), (6, 3, 128, 384, 128)])
 def test_int4_rope_kv_matches_two_kernel_path_and_stock_ops(bsz, n_head, n_kv, d, k, g):
     from easy_to_hard_amd.model import apply_rotary_emb, precompute_freqs_cis
 
-    if k == 4096 and bsz not in (1, 32):
-        pytest.skip("large shape: first and last batch size only")
+    if k == 4096 and bsz not in (1, 32, 64):
+        pytest.skip("large shape: three batch sizes only")
     n = (n_head + 2 * n_kv) * d
     s_max, pos = 80, 37
     codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=n + bsz)
