@@ -133,7 +133,7 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
     const uint32_t *__restrict__ wp2, const uint32_t *__restrict__ sz2,
     uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K,
-    RopeArgs rope) {
+    int slabs_in_x, RopeArgs rope) {
   constexpr bool GATE = EPI == kGate;
   static_assert(EPI != kRope || T == 1, "the rotary epilogue handles one column tile per wave");
   static_assert(!GATE || T == 2, "gate mode pairs exactly two weight matrices");
@@ -181,8 +181,18 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   const int c1 = C0 + ((C1 - C0) * (kg + 1)) / WK;
   const int nloc = c1 - c0;
   const int nloc_max = (C1 - C0 + WK - 1) / WK;  // trip count, uniform over the workgroup
-  const int tile16_0 = (blockIdx.x * kWavesN + wave_n) * TC;
-  const int m_base = blockIdx.z * (16 * MT);
+  // Column block and row slab of this workgroup.  A few row slabs (decode batches of 33 .. 128 rows) are folded into
+  // blockIdx.x so that the slabs of one column block are dispatched together AND land on the same XCD (workgroup
+  // i goes to XCD i % 8): the second slab then finds the weights in that XCD's L2 instead of fetching them again.
+  const int n_blocks = ((N + 15) / 16 + kWavesN * TC - 1) / (kWavesN * TC);
+  int col_block = blockIdx.x, row_slab = blockIdx.z;
+  if (slabs_in_x > 1) {
+    row_slab = (blockIdx.x >> 3) % slabs_in_x;
+    col_block = (blockIdx.x / (8 * slabs_in_x)) * 8 + (blockIdx.x & 7);
+    if (col_block >= n_blocks) return;  // padding of the folded grid; uniform over the workgroup, before any barrier
+  }
+  const int tile16_0 = (col_block * kWavesN + wave_n) * TC;
+  const int m_base = row_slab * (16 * MT);
   uint8_t *const xlds = lds + kg * (2 * kStageBytes);
 
   // ---- addressing: uniform (scalar) base per chunk + constant 32-bit per-lane byte offsets ------------
@@ -415,7 +425,7 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   // ticket is taken, and the loads are issued after it has been observed.
   if (S > 1) {
     const size_t tile_floats = static_cast<size_t>(kWavesN) * kSlots * 64;
-    const size_t wg_tile = static_cast<size_t>(blockIdx.z) * gridDim.x + blockIdx.x;
+    const size_t wg_tile = static_cast<size_t>(row_slab) * n_blocks + col_block;
     if (kg == 0) {
       float *mine = ws_partial + (wg_tile * S + ks) * tile_floats + static_cast<size_t>(wave_n) * kSlots * 64 + lane;
 #pragma unroll
@@ -528,11 +538,15 @@ template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain>
 int launch(const LaunchArgs &a) {
   const int tiles16 = (a.N + 15) / 16;
   constexpr int TC = EPI == kGate ? 1 : T;
-  dim3 grid((tiles16 + WN * TC - 1) / (WN * TC), a.S, (a.M + 16 * MT - 1) / (16 * MT));
+  const int n_blocks = (tiles16 + WN * TC - 1) / (WN * TC);
+  const int m_chunks = (a.M + 16 * MT - 1) / (16 * MT);
+  const int slabs_in_x = (m_chunks > 1 && m_chunks <= 4) ? m_chunks : 1;
+  dim3 grid(n_blocks, a.S, m_chunks);
+  if (slabs_in_x > 1) grid = dim3(((n_blocks + 7) / 8) * 8 * slabs_in_x, a.S, 1);
   hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK, EPI>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
                      reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz),
                      reinterpret_cast<const uint32_t *>(a.packed2), reinterpret_cast<const uint32_t *>(a.sz2), a.y,
-                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K, a.rope);
+                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K, slabs_in_x, a.rope);
   return launch_status();
 }
 
