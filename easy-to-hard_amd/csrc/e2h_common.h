@@ -15,7 +15,7 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kWaveSize = 64;
 
-// ---- bfloat16 <-> float32 (bit exact, round to nearest even; NaN inputs are not expected) --------
+// ---- bfloat16 <-> float32 (bit exact, round to nearest even; NaN stays a quiet NaN) -----------------
 
 __host__ __device__ inline float bf16_to_f32(uint16_t b) {
   uint32_t u = static_cast<uint32_t>(b) << 16;
@@ -24,6 +24,7 @@ __host__ __device__ inline float bf16_to_f32(uint16_t b) {
 
 __host__ __device__ inline uint16_t f32_to_bf16_rne(float f) {
   uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);  // the rounding add would carry a NaN away
   u += 0x7FFFu + ((u >> 16) & 1u);
   return static_cast<uint16_t>(u >> 16);
 }

@@ -334,3 +334,20 @@ def test_int4_rope_kv_ignores_out_of_range_position():
     ops.int4_mm_rope_kv(x, packed_d, sz_d, g, freqs, kc, vc, torch.tensor([s_max], device=DEV), n_head, n_kv, d)
     torch.cuda.synchronize()
     assert torch.equal(kc, kc0) and torch.equal(vc, kc0)
+
+
+def test_nan_and_inf_activations_propagate_to_their_rows_only():
+    """A NaN / inf in one row of x must show up as NaN / inf in that row's outputs (torch semantics) and nowhere else."""
+    codes, sz, packed_d, sz_d = _int4_case(64, 512, 128, 8)
+    x = randn_bf16((8, 512), seed=9)
+    x[2, 100] = float("nan")
+    x[5, 7] = float("inf")
+    y = ops.int4_mm_direct(x.to(DEV), packed_d, 128, sz_d).float().cpu()
+    assert torch.isnan(y[2]).all()
+    assert not torch.isfinite(y[5]).any()
+    keep = [0, 1, 3, 4, 6, 7]
+    assert torch.isfinite(y[keep]).all()
+    q = torch.randint(-128, 128, (64, 512), dtype=torch.int8).to(DEV)
+    s = torch.ones(64, dtype=torch.bfloat16, device=DEV)
+    y8 = ops.int8_mm_direct(x.to(DEV), q, s).float().cpu()
+    assert torch.isnan(y8[2]).all() and not torch.isfinite(y8[5]).any() and torch.isfinite(y8[keep]).all()
