@@ -64,6 +64,10 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.int8_k_slices = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "int4_no_xsum")) {
+    o.int4_no_xsum = value != 0;
+    return E2H_OK;
+  }
   if (!strcmp(name, "row_tiles")) {
     if (value != 0 && value != 1 && value != 2 && value != 4) return E2H_ERR_BAD_OPTION;
     o.row_tiles = value;

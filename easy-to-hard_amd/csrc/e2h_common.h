@@ -43,6 +43,7 @@ struct Options {
   int int8_k_groups;       // 0 = heuristic, else 1/2
   int int8_k_slices;       // 0 = heuristic, else 1..16
   int int8_force_generic;  // 1 = always use the generic (bounds-checked) int8 kernel
+  int int4_no_xsum;        // 1 = many-row int4 calls compute the group sums of x inside the matmul (no pre-pass)
   int row_tiles;           // 0 = heuristic, else 1/2/4 tiles of 16 activation rows per workgroup (both matmuls)
 };
 Options &options();

@@ -54,11 +54,12 @@ template <> struct WordVec<4> { typedef u32x4_t type; };
 
 constexpr int kFragBytes = 1024 + 64;   // one MFMA A-fragment block in LDS; the pad skews banks between steps
 
-template <int G, int IKT, int T>
+template <int G, int IKT, int T, int XS>
 struct WeightRegs {
   typedef Int4Geom<G, IKT> Geo;
   uint32_t w[T][Geo::STEPS];
   uint32_t sz[T][Geo::NGRP];
+  f32x4_t xs[XS > 0 ? XS : 1][Geo::NGRP];  // precomputed group sums of x for the chunk (XS = row tiles), else unused
 };
 
 constexpr int kWeightCachePolicy = 2;  // "nt": weights are streamed once, keep them from displacing x and qparams
@@ -128,18 +129,18 @@ struct RopeArgs {
   int H, Hkv, S, D;
 };
 
-template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain>
+template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain, bool XSUM = false>
 __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp, const uint32_t *__restrict__ sz,
     const uint32_t *__restrict__ wp2, const uint32_t *__restrict__ sz2,
     uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K,
-    int slabs_in_x, RopeArgs rope) {
+    int slabs_in_x, RopeArgs rope, const float *__restrict__ xsum, int xsum_stride) {
   constexpr bool GATE = EPI == kGate;
   static_assert(EPI != kRope || T == 1, "the rotary epilogue handles one column tile per wave");
   static_assert(!GATE || T == 2, "gate mode pairs exactly two weight matrices");
   constexpr int TC = GATE ? 1 : T;  // distinct column tiles per wave
   typedef Int4Geom<G, IKT> Geo;
-  typedef WeightRegs<G, IKT, T> wregs_t;
+  typedef WeightRegs<G, IKT, T, XSUM ? MT : 0> wregs_t;
   constexpr int kWavesN = WN;
   constexpr int kGroupThreads = WN * 64;
   constexpr int NB = Tuning<G, IKT, MT, T, WN, WK>::NB;
@@ -214,6 +215,10 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   const __amdgpu_buffer_rsrc_t sz_rsrc = make_rsrc(sz, static_cast<uint32_t>(static_cast<size_t>(K / G) * N * 4));
   const __amdgpu_buffer_rsrc_t w2_rsrc = make_rsrc(GATE ? wp2 : wp, static_cast<uint32_t>(static_cast<size_t>(N) * K / 2));
   const __amdgpu_buffer_rsrc_t sz2_rsrc = make_rsrc(GATE ? sz2 : sz, static_cast<uint32_t>(static_cast<size_t>(K / G) * N * 4));
+  // XSUM: the sums of x over every (row, quantization group) were computed once by a pre-pass, laid out
+  // [K/G][xsum_stride] float32; each lane fetches the four rows of its accumulator registers per row tile
+  const __amdgpu_buffer_rsrc_t xs_rsrc = make_rsrc(XSUM ? xsum : reinterpret_cast<const float *>(x),
+                                                   XSUM ? static_cast<uint32_t>(static_cast<size_t>(K / G) * xsum_stride * 4) : 0u);
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
 
   auto load_weights = [&](wregs_t &r, int ci) {
@@ -241,6 +246,16 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
 #pragma unroll
       for (int g = 0; g < Geo::NGRP; ++g)
         r.sz[t][g] = __builtin_amdgcn_raw_buffer_load_b32(sr, szlane[t], szchunk + g * N * 4, 0);
+    }
+    if constexpr (XSUM) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int g = 0; g < Geo::NGRP; ++g) {
+          const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(
+              xs_rsrc, static_cast<uint32_t>((m_base + 16 * mt + 4 * b) * 4), static_cast<uint32_t>(ci * Geo::NGRP + g) * static_cast<uint32_t>(xsum_stride) * 4u, 0);
+          r.xs[mt][g] = __builtin_bit_cast(f32x4_t, v);
+        }
     }
   };
 
@@ -308,11 +323,15 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
       for (int g = 0; g < Geo::NGRP; ++g) {
-        f32x4_t s4 = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (XSUM) {
+          xs[mt][g] = r.xs[mt][g];
+        } else {
+          f32x4_t s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < Geo::SPG; ++s)
-          s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][g * Geo::SPG + s], ones, s4, 0, 0, 0);
-        xs[mt][g] = s4;
+          for (int s = 0; s < Geo::SPG; ++s)
+            s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[mt][g * Geo::SPG + s], ones, s4, 0, 0, 0);
+          xs[mt][g] = s4;
+        }
       }
     }
 #pragma unroll
@@ -520,6 +539,25 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   }
 }
 
+// Pre-pass for many-row calls: sums of x over every (row, quantization group), float32, stored group-major
+// [K/G][stride] so that the matmul's lanes read four consecutive rows with one 16-byte load.  Reads x once
+// (2 M K bytes); the matmul then needs no arithmetic at all for the zero-point term's x side.
+template <int G>
+__global__ __launch_bounds__(256) void x_group_sums_kernel(const uint16_t *__restrict__ x, float *__restrict__ out, int M, int K, int stride) {
+  constexpr int PG = G / 8;  // 16-byte pieces per group (4 .. 32 lanes of one wave)
+  const int m = blockIdx.x;
+  const uint16_t *row = x + static_cast<size_t>(m) * K;
+  for (int piece = threadIdx.x; piece < K / 8; piece += 256) {  // K % G == 0, so whole groups stay inside one wave's lanes
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(row + piece * 8);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s += __builtin_bit_cast(float, raw[j] << 16) + __builtin_bit_cast(float, raw[j] & 0xFFFF0000u);
+#pragma unroll
+    for (int off = 1; off < PG; off <<= 1) s += __shfl_xor(s, off);
+    if ((piece % PG) == 0) out[static_cast<size_t>(piece / PG) * stride + m] = s;
+  }
+}
+
 struct LaunchArgs {
   const uint16_t *x;
   const int32_t *packed;
@@ -528,13 +566,15 @@ struct LaunchArgs {
   const uint16_t *sz2;
   uint16_t *y;
   RopeArgs rope;
+  const float *xsum;  // group sums of x from the pre-pass (large M), else null
+  int xsum_stride;
   float *ws_partial;
   unsigned *ws_ticket;
   int M, N, K, S;
   hipStream_t stream;
 };
 
-template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain>
+template <int G, int IKT, int MT, int T, int WN, int WK, int EPI = kPlain, bool XSUM = false>
 int launch(const LaunchArgs &a) {
   const int tiles16 = (a.N + 15) / 16;
   constexpr int TC = EPI == kGate ? 1 : T;
@@ -543,10 +583,10 @@ int launch(const LaunchArgs &a) {
   const int slabs_in_x = (m_chunks > 1 && m_chunks <= 4) ? m_chunks : 1;
   dim3 grid(n_blocks, a.S, m_chunks);
   if (slabs_in_x > 1) grid = dim3(((n_blocks + 7) / 8) * 8 * slabs_in_x, a.S, 1);
-  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK, EPI>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
+  hipLaunchKernelGGL((int4_skinny_mm_kernel<G, IKT, MT, T, WN, WK, EPI, XSUM>), grid, dim3(64 * WN * WK), 0, a.stream, a.x,
                      reinterpret_cast<const uint32_t *>(a.packed), reinterpret_cast<const uint32_t *>(a.sz),
                      reinterpret_cast<const uint32_t *>(a.packed2), reinterpret_cast<const uint32_t *>(a.sz2), a.y,
-                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K, slabs_in_x, a.rope);
+                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K, slabs_in_x, a.rope, a.xsum, a.xsum_stride);
   return launch_status();
 }
 
@@ -568,6 +608,10 @@ int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
     E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 4, 4) E2H_CASE(1, 3, 4) E2H_CASE(1, 2, 4) E2H_CASE(1, 2, 2)
     E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1)
 #undef E2H_CASE
+    if (a.xsum) {
+      if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1, kPlain, true>(a);
+      if (sh.t == 1) return launch<G, IKT, 4, 1, 4, 1, kPlain, true>(a);
+    }
     if (sh.t == 4) return launch<G, IKT, 4, 4, 4, 1>(a);
     if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1>(a);
     return launch<G, IKT, 4, 1, 4, 1>(a);
@@ -616,7 +660,7 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
   LaunchArgs a;
   a.x = x; a.packed = packed; a.sz = scales_and_zeros; a.y = y;
-  a.packed2 = nullptr; a.sz2 = nullptr; a.rope = RopeArgs{};
+  a.packed2 = nullptr; a.sz2 = nullptr; a.rope = RopeArgs{}; a.xsum = nullptr; a.xsum_stride = 0;
   a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
   a.stream = static_cast<hipStream_t>(stream);
   // up to 64 rows (decode batches): 32-row workgroups with the K-split shapes, two row slabs per column block
@@ -681,6 +725,23 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     a.x = x + m0 * a.K;
     a.y = y + m0 * a.N;
     a.M = static_cast<int>(m_total - m0 < max_rows ? m_total - m0 : max_rows);
+    a.xsum = nullptr;
+    if (mt == 4 && wide_ok && (sh.t == 1 || sh.t == 2) && workspace && !options().int4_no_xsum) {
+      // many rows: one pass over x leaves its group sums in the workspace's partial-tile area (unused here: no K split)
+      const int stride = ((a.M + 63) / 64) * 64;
+      const int64_t need = static_cast<int64_t>(kTicketBytes) + static_cast<int64_t>(a.K / groupsize) * stride * 4;
+      if (need <= workspace_bytes) {
+        float *xs = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + kTicketBytes);
+        switch (groupsize) {
+          case 32: hipLaunchKernelGGL(x_group_sums_kernel<32>, dim3(a.M), dim3(256), 0, a.stream, a.x, xs, a.M, a.K, stride); break;
+          case 64: hipLaunchKernelGGL(x_group_sums_kernel<64>, dim3(a.M), dim3(256), 0, a.stream, a.x, xs, a.M, a.K, stride); break;
+          default: hipLaunchKernelGGL(x_group_sums_kernel<128>, dim3(a.M), dim3(256), 0, a.stream, a.x, xs, a.M, a.K, stride); break;
+        }
+        if (launch_status() != E2H_OK) return E2H_ERR_LAUNCH;
+        a.xsum = xs;
+        a.xsum_stride = stride;
+      }
+    }
     int rc;
     switch (groupsize) {
       case 32: rc = dispatch_ikt<32>(inner_k_tiles, mt, sh, a); break;
@@ -725,7 +786,7 @@ extern "C" int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_ga
   LaunchArgs a;
   a.x = x; a.packed = packed_gate; a.sz = sz_gate; a.packed2 = packed_up; a.sz2 = sz_up; a.y = y;
   a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
-  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr; a.rope = RopeArgs{};
+  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr; a.rope = RopeArgs{}; a.xsum = nullptr; a.xsum_stride = 0;
   a.stream = static_cast<hipStream_t>(stream);
   const int mt = a.M <= 16 ? 1 : 2;
   // column waves per workgroup: the count that leaves the fewest idle CUs in the last round of workgroups
@@ -775,7 +836,7 @@ extern "C" int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, con
   a.rope = RopeArgs{freqs_cis, q_out, k_cache, v_cache, input_pos, static_cast<int>(n_head), static_cast<int>(n_kv_head),
                     static_cast<int>(cache_len), static_cast<int>(head_dim)};
   a.M = static_cast<int>(batch); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
-  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr;
+  a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr; a.xsum = nullptr; a.xsum_stride = 0;
   a.stream = static_cast<hipStream_t>(stream);
   const bool two = a.M > 16;
   switch (groupsize) {

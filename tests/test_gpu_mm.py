@@ -351,3 +351,21 @@ def test_nan_and_inf_activations_propagate_to_their_rows_only():
     s = torch.ones(64, dtype=torch.bfloat16, device=DEV)
     y8 = ops.int8_mm_direct(x.to(DEV), q, s).float().cpu()
     assert torch.isnan(y8[2]).all() and not torch.isfinite(y8[5]).any() and torch.isfinite(y8[keep]).all()
+
+
+@pytest.mark.parametrize("g", [32, 64, 128])
+@pytest.mark.parametrize("m", [65, 130, 257])
+def test_int4_many_rows_group_sum_prepass_matches_in_kernel_sums(m, g):
+    """Calls with more than 64 rows take the group sums of x from a pre-pass; the in-kernel form (option
+    int4_no_xsum) must agree to float32 summation-order noise, and both with the oracle."""
+    n, k = 272, 1024
+    codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=m + g)
+    x = randn_bf16((m, k), std=1.0, seed=m)
+    y, _ = _check_int4(x, codes, sz, packed_d, sz_d, g)
+    _lib.set_option("int4_no_xsum", 1)
+    try:
+        y2, _ = _check_int4(x, codes, sz, packed_d, sz_d, g)
+    finally:
+        _lib.set_option("int4_no_xsum", 0)
+    diff = (y.float() - y2.float()).abs().max().item()
+    assert diff <= 2.0 ** -7 * y2.float().abs().max().item()  # at most one bf16 step of the largest output
