@@ -1,7 +1,8 @@
 """Batched greedy decoding and reward scoring on top of model.Transformer (harness for the decode configs).
 
 Follows the control flow of the reference's inference_generate.py (`prefill` :98-107, `decode_one_token`
-:110-120, `decode_n_tokens` :123-157, `generate` :164-221) with greedy argmax in place of sampling, and of
+:110-120, `decode_n_tokens` :123-157, `generate` :164-221) with greedy argmax by default and the reference's
+temperature / top-k sampling (`sample` :72-85) on request, and of
 inference_reward.py `model_score` (:67-91).  The decode step can be captured once into a HIP graph and
 replayed per token: every kernel of this package enqueues on the current stream with a launch geometry
 that depends on shapes only.
@@ -12,28 +13,68 @@ from typing import Optional
 import torch
 from torch import Tensor
 
+from . import ops
+
 
 def greedy_token(logits: Tensor) -> Tensor:
     """argmax over the vocabulary of the last position, in float32 -> [B, 1] int64."""
     return torch.argmax(logits[:, -1].float(), dim=-1, keepdim=True)
 
 
-@torch.no_grad()
-def prefill(model, x: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None) -> Tensor:
-    return greedy_token(model(x, input_pos, left_pad_mask_pos))
+def multinomial_sample_one_no_sync(probs_sort: Tensor) -> Tensor:
+    """reference inference_generate.py:53-58: exponential race, no host synchronisation."""
+    q = torch.empty_like(probs_sort).exponential_(1)
+    return torch.argmax(probs_sort / q, dim=-1, keepdim=True).to(dtype=torch.int)
+
+
+def logits_to_probs(logits: Tensor, temperature: float = 1.0, top_k: Optional[int] = None) -> Tensor:
+    """reference inference_generate.py:61-69 with stock ops (used for inputs the fused kernel does not take)."""
+    logits = logits / max(temperature, 1e-5)
+    if top_k is not None:
+        v, _ = torch.topk(logits, min(top_k, logits.size(-1)), dim=-1)
+        pivot = v.select(-1, -1).view(-1, 1)
+        logits = torch.where(logits < pivot, -float("Inf"), logits)
+    return torch.nn.functional.softmax(logits, dim=-1)
+
+
+def sample(logits: Tensor, temperature: float = 1.0, top_k: Optional[int] = None):
+    """reference inference_generate.py:72-85 (one GPU, so no vocab-parallel gather): logits [B, S, V] ->
+    (idx_next int32 [B, 1], probs float32 [B, V]) for the last position.  bfloat16 logits on the GPU take the
+    fused kernel; the Exp(1) draws come from torch's generator exactly as in the reference."""
+    last = logits[:, -1]
+    if last.is_cuda and last.dtype == torch.bfloat16:
+        q = torch.empty(last.shape, dtype=torch.float32, device=last.device).exponential_(1)
+        return ops.sample_top_k(last, q, temperature, top_k)
+    probs = logits_to_probs(last.float(), temperature, top_k)
+    return multinomial_sample_one_no_sync(probs), probs
+
+
+def _next_token(logits: Tensor, temperature: Optional[float], top_k: Optional[int]) -> Tensor:
+    if temperature is None:
+        return greedy_token(logits)
+    return sample(logits, temperature, top_k)[0].to(torch.int64)
 
 
 @torch.no_grad()
-def decode_one_token(model, cur_token: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None) -> Tensor:
+def prefill(model, x: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None,
+            temperature: Optional[float] = None, top_k: Optional[int] = None) -> Tensor:
+    """temperature None = greedy arg-max, else the reference's sampling."""
+    return _next_token(model(x, input_pos, left_pad_mask_pos), temperature, top_k)
+
+
+@torch.no_grad()
+def decode_one_token(model, cur_token: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None,
+                     temperature: Optional[float] = None, top_k: Optional[int] = None) -> Tensor:
     assert input_pos.shape[-1] == 1
-    return greedy_token(model(cur_token, input_pos, left_pad_mask_pos))
+    return _next_token(model(cur_token, input_pos, left_pad_mask_pos), temperature, top_k)
 
 
 class GraphedDecodeStep:
     """One decode step captured into a HIP graph; `step(token, pos)` copies the inputs into the static
     buffers, replays the graph and returns the static output buffer ([B, 1] next tokens)."""
 
-    def __init__(self, model, batch_size: int, device, left_pad_mask_pos: Optional[Tensor] = None, warmup: int = 2):
+    def __init__(self, model, batch_size: int, device, left_pad_mask_pos: Optional[Tensor] = None, warmup: int = 2,
+                 temperature: Optional[float] = None, top_k: Optional[int] = None):
         self.model = model
         self.cur_token = torch.zeros((batch_size, 1), dtype=torch.int64, device=device)
         self.input_pos = torch.zeros((1,), dtype=torch.int64, device=device)
@@ -42,11 +83,11 @@ class GraphedDecodeStep:
         side.wait_stream(torch.cuda.current_stream(device))
         with torch.cuda.stream(side):
             for _ in range(warmup):
-                decode_one_token(model, self.cur_token, self.input_pos, self.left_pad)
+                decode_one_token(model, self.cur_token, self.input_pos, self.left_pad, temperature, top_k)
         torch.cuda.current_stream(device).wait_stream(side)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            self.next_token = decode_one_token(model, self.cur_token, self.input_pos, self.left_pad)
+            self.next_token = decode_one_token(model, self.cur_token, self.input_pos, self.left_pad, temperature, top_k)
 
     def step(self, cur_token: Tensor, input_pos: Tensor) -> Tensor:
         self.cur_token.copy_(cur_token)
@@ -57,8 +98,10 @@ class GraphedDecodeStep:
 
 @torch.no_grad()
 def generate(model, prompt: Tensor, max_new_tokens: int, use_graph: bool = True,
-             left_pad_mask_pos: Optional[Tensor] = None, stepper: Optional[GraphedDecodeStep] = None) -> Tensor:
-    """prompt [B, T] int64 on the GPU -> [B, T + max_new_tokens] (prompt followed by greedy tokens)."""
+             left_pad_mask_pos: Optional[Tensor] = None, stepper: Optional[GraphedDecodeStep] = None,
+             temperature: Optional[float] = None, top_k: Optional[int] = None) -> Tensor:
+    """prompt [B, T] int64 on the GPU -> [B, T + max_new_tokens] (prompt followed by the new tokens: greedy when
+    temperature is None, else sampled as the reference does, inference_generate.py:123-221)."""
     bsz, t = prompt.shape
     total = t + max_new_tokens
     device = prompt.device
@@ -66,19 +109,20 @@ def generate(model, prompt: Tensor, max_new_tokens: int, use_graph: bool = True,
     seq = torch.empty((bsz, total), dtype=prompt.dtype, device=device)
     seq[:, :t] = prompt
     input_pos = torch.arange(0, t, device=device)
-    cur = prefill(model, prompt, input_pos, left_pad_mask_pos)
+    cur = prefill(model, prompt, input_pos, left_pad_mask_pos, temperature, top_k)
     seq[:, t] = cur[:, 0]
     if max_new_tokens > 1:
         if use_graph and stepper is None:
-            stepper = GraphedDecodeStep(model, bsz, device, left_pad_mask_pos)
+            stepper = GraphedDecodeStep(model, bsz, device, left_pad_mask_pos, temperature=temperature, top_k=top_k)
             # the capture warm-up wrote garbage K/V at position 0 of the cache: recompute the prompt
-            cur = prefill(model, prompt, input_pos, left_pad_mask_pos)
+            cur = prefill(model, prompt, input_pos, left_pad_mask_pos, temperature, top_k)
+            seq[:, t] = cur[:, 0]
         pos = torch.tensor([t], device=device, dtype=torch.int64)
         for i in range(1, max_new_tokens):
             if stepper is not None:
                 cur = stepper.step(cur, pos).clone()
             else:
-                cur = decode_one_token(model, cur, pos, left_pad_mask_pos)
+                cur = decode_one_token(model, cur, pos, left_pad_mask_pos, temperature, top_k)
             seq[:, t + i] = cur[:, 0]
             pos += 1
     return seq

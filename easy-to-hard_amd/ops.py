@@ -434,6 +434,24 @@ def int4_mm_rope_kv(x, packed, scales_and_zeros, groupsize, freqs_cis, k_cache, 
     return q
 
 
+def sample_top_k(logits, q, temperature=1.0, top_k=None):
+    """logits bf16 [B, V] (rows may be strided), q float32 [B, V] of Exp(1) draws -> (idx int32 [B, 1], probs float32 [B, V]):
+    softmax(top-k-masked logits / max(temperature, 1e-5)) and argmax(probs / q), in one launch."""
+    _need_gpu(logits, q)
+    assert logits.dtype == torch.bfloat16 and logits.dim() == 2 and q.dtype == torch.float32 and q.shape == logits.shape
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    q = q.contiguous()
+    rows, vocab = logits.shape
+    probs = torch.empty((rows, vocab), dtype=torch.float32, device=logits.device)
+    idx = torch.empty((rows, 1), dtype=torch.int32, device=logits.device)
+    k = 0 if top_k is None else min(int(top_k), vocab)
+    rc = _lib_for(logits).e2h_sample_top_k(_ptr(logits), logits.stride(0), _ptr(q), _ptr(probs), _ptr(idx), rows, vocab,
+                                          float(temperature), k, _stream(logits))
+    _lib.check(rc, "e2h_sample_top_k")
+    return idx, probs
+
+
 def decode_attention(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, scale=None):
     """q bf16 [B, H, D] against caches [Bmax, Hkv, S, D] up to and including input_pos -> bf16 [B, H, D]."""
     _need_gpu(q, k_cache, v_cache, input_pos)

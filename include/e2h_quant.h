@@ -193,6 +193,16 @@ int e2h_rope_kv_write(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *
 /* F.silu(a) * b with bf16 rounding after each op (reference FeedForward.forward :359-360). n elements, n % 8 == 0. */
 int e2h_silu_mul(const uint16_t *a, const uint16_t *b, uint16_t *y, int64_t n, void *stream);
 
+/* Next-token sampling, reference inference_generate.py:53-85 (sample -> logits_to_probs ->
+ * multinomial_sample_one_no_sync) on the last position's logits:
+ *   l = float(logits) / max(temperature, 1e-5);  with top_k > 0: l = (l < k-th largest l of the row) ? -inf : l;
+ *   probs = softmax(l);  idx = argmax(probs / q).
+ *   logits [rows, >= vocab] bf16 with row_stride elements between rows; q [rows, vocab] float32, the Exp(1) draws
+ *   (the caller makes them, as the reference does with exponential_(1)); probs [rows, vocab] float32 out;
+ *   idx [rows] int32 out.  top_k == 0 or top_k >= vocab: no truncation.  Ties at the pivot all survive. */
+int e2h_sample_top_k(const uint16_t *logits, int64_t row_stride, const float *q, float *probs, int32_t *idx,
+                     int64_t rows, int64_t vocab, float temperature, int top_k, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
