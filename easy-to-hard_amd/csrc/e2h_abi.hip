@@ -68,6 +68,15 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.int4_no_xsum = value != 0;
     return E2H_OK;
   }
+  if (!strcmp(name, "int4_no_gemm32")) {
+    o.int4_no_gemm32 = value != 0;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int4_gemm32_min_rows")) {
+    if (value < 0) return E2H_ERR_BAD_OPTION;
+    o.int4_gemm32_min_rows = value;
+    return E2H_OK;
+  }
   if (!strcmp(name, "row_tiles")) {
     if (value != 0 && value != 1 && value != 2 && value != 4) return E2H_ERR_BAD_OPTION;
     o.row_tiles = value;

@@ -31,6 +31,7 @@
 // float32 partial tile, takes a ticket, and the last one to arrive adds the S partials in slice order -- a
 // fixed order, so results are deterministic -- and writes bf16.
 #include "e2h_common.h"
+#include "e2h_int4_unpack.h"
 
 namespace e2h {
 namespace {
@@ -64,28 +65,6 @@ struct WeightRegs {
 
 constexpr int kWeightCachePolicy = 2;  // "nt": weights are streamed once, keep them from displacing x and qparams
 
-
-// (w >> 4i) & 0x000F000F | 0x43004300: two codes -> the bfloat16 pair (128 + q, 128 + q').  The mask lives
-// in an SGPR and the magic in a VGPR so that each pair is one v_and_or_b32 (this ISA's VOP3 encoding takes no
-// literal and only one scalar operand); the asm statements only keep the compiler from folding them back
-// into literals.
-struct UnpackConsts {
-  uint32_t mask, magic;
-};
-__device__ __forceinline__ UnpackConsts unpack_consts() {
-  UnpackConsts c;
-  asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(c.mask));
-  asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(c.magic));
-  return c;
-}
-__device__ __forceinline__ bf16x8_t unpack_word(uint32_t w, const UnpackConsts &c) {
-  u32x4_t u;
-  u[0] = (w & c.mask) | c.magic;
-  u[1] = ((w >> 4) & c.mask) | c.magic;
-  u[2] = ((w >> 8) & c.mask) | c.magic;
-  u[3] = ((w >> 12) & c.mask) | c.magic;
-  return __builtin_bit_cast(bf16x8_t, u);
-}
 
 // Weight prefetch: a ring of NB register buffers per wave, NB - 1 chunks in flight beyond the one being
 // consumed (about 8 KB per wave: HBM latency here is well over a microsecond, so a CU needs tens of KB in
@@ -642,6 +621,18 @@ constexpr int kCUs = 256;
 }  // namespace
 }  // namespace e2h
 
+namespace e2h {
+int launch_x_group_sums(const uint16_t *x, float *out, int M, int K, int stride, int groupsize, hipStream_t stream) {
+  switch (groupsize) {
+    case 32: hipLaunchKernelGGL(x_group_sums_kernel<32>, dim3(M), dim3(256), 0, stream, x, out, M, K, stride); break;
+    case 64: hipLaunchKernelGGL(x_group_sums_kernel<64>, dim3(M), dim3(256), 0, stream, x, out, M, K, stride); break;
+    case 128: hipLaunchKernelGGL(x_group_sums_kernel<128>, dim3(M), dim3(256), 0, stream, x, out, M, K, stride); break;
+    default: return E2H_ERR_BAD_GROUPSIZE;
+  }
+  return launch_status();
+}
+}  // namespace e2h
+
 extern "C" int64_t e2h_workspace_bytes(void) { return static_cast<int64_t>(e2h::kTicketBytes) + (int64_t{32} << 20); }
 
 extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
@@ -732,14 +723,16 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
       const int64_t need = static_cast<int64_t>(kTicketBytes) + static_cast<int64_t>(a.K / groupsize) * stride * 4;
       if (need <= workspace_bytes) {
         float *xs = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + kTicketBytes);
-        switch (groupsize) {
-          case 32: hipLaunchKernelGGL(x_group_sums_kernel<32>, dim3(a.M), dim3(256), 0, a.stream, a.x, xs, a.M, a.K, stride); break;
-          case 64: hipLaunchKernelGGL(x_group_sums_kernel<64>, dim3(a.M), dim3(256), 0, a.stream, a.x, xs, a.M, a.K, stride); break;
-          default: hipLaunchKernelGGL(x_group_sums_kernel<128>, dim3(a.M), dim3(256), 0, a.stream, a.x, xs, a.M, a.K, stride); break;
-        }
-        if (launch_status() != E2H_OK) return E2H_ERR_LAUNCH;
+        if (launch_x_group_sums(a.x, xs, a.M, a.K, stride, groupsize, a.stream) != E2H_OK) return E2H_ERR_LAUNCH;
         a.xsum = xs;
         a.xsum_stride = stride;
+        // 32x32-tile kernel for whole 128-row blocks' worth of work
+        const int min32 = options().int4_gemm32_min_rows > 0 ? options().int4_gemm32_min_rows : 256;
+        if (a.M >= min32 && !options().int4_no_gemm32) {
+          const int rc32 = int4_gemm32(a.x, a.packed, a.sz, a.y, xs, stride, a.M, a.N, a.K, groupsize, a.stream);
+          if (rc32 != E2H_OK) return rc32;
+          continue;
+        }
       }
     }
     int rc;

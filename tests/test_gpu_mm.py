@@ -369,3 +369,30 @@ def test_int4_many_rows_group_sum_prepass_matches_in_kernel_sums(m, g):
         _lib.set_option("int4_no_xsum", 0)
     diff = (y.float() - y2.float()).abs().max().item()
     assert diff <= 2.0 ** -7 * y2.float().abs().max().item()  # at most one bf16 step of the largest output
+
+
+@pytest.mark.parametrize("g", [32, 64, 128])
+@pytest.mark.parametrize("m,n,k", [(65, 8, 128), (130, 272, 1024), (257, 136, 384), (512, 4096, 4096)])
+def test_int4_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, g):
+    """The 32x32-tile kernel (many rows) against the oracle and against the 16x16-tile kernel on the same inputs:
+    ragged M and N (not multiples of 128 / 32), a single chunk, odd numbers of groups."""
+    if k == 4096 and g != 128:
+        pytest.skip("large shape: one group size only")
+    codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=m + n + g)
+    x = randn_bf16((m, k), std=1.0, seed=m + 1)
+    _lib.set_option("int4_gemm32_min_rows", 65)
+    try:
+        y, _ = _check_int4(x, codes, sz, packed_d, sz_d, g)
+        # exact small-integer case: x in {-1, 0, 1}, every partial sum is an integer well inside float32
+        xi = torch.randint(-1, 2, (m, k), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+        yi = ops.int4_mm_direct(xi.to(DEV), packed_d, g, sz_d)
+    finally:
+        _lib.set_option("int4_gemm32_min_rows", 0)
+    _lib.set_option("int4_no_gemm32", 1)
+    try:
+        y2, _ = _check_int4(x, codes, sz, packed_d, sz_d, g)
+        yi2 = ops.int4_mm_direct(xi.to(DEV), packed_d, g, sz_d)
+    finally:
+        _lib.set_option("int4_no_gemm32", 0)
+    assert (y.float() - y2.float()).abs().max().item() <= 2.0 ** -7 * y2.float().abs().max().item()
+    assert (yi.float() - yi2.float()).abs().max().item() <= 2.0 ** -7 * yi2.float().abs().max().item()
