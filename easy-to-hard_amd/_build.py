@@ -32,6 +32,12 @@ HIPCC_FLAGS = [
 ]
 
 
+# Per-source additions.  The 32x32-tile matmul mixes MFMA accumulators with float32 FMAs on the same values; with
+# the accumulators in the accumulation register file every FMA needs copies in and out (3 extra instructions per FMA),
+# so that file is compiled with MFMA results kept in ordinary vector registers.
+EXTRA_FLAGS = {"e2h_int4_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _hipcc():
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and Path(cand).exists():
@@ -55,7 +61,7 @@ def build_library(verbose=False):
 
     def compile_one(src):
         obj = obj_dir / (Path(src).stem + ".o")
-        out = _run([hipcc, *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)])
+        out = _run([hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-c", str(CSRC / src), "-o", str(obj)])
         if verbose and out.strip():
             print(out)
         return obj
