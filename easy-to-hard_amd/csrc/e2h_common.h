@@ -44,7 +44,7 @@ struct Options {
   int int8_k_slices;       // 0 = heuristic, else 1..16
   int int8_force_generic;  // 1 = always use the generic (bounds-checked) int8 kernel
   int int4_no_xsum;        // 1 = many-row int4 calls compute the group sums of x inside the matmul (no pre-pass)
-  int int4_no_gemm32;      // 1 = many-row int4 calls stay on the 16x16-tile kernel
+  int int4_no_gemm32;      // 1 = many-row calls (int4 and int8) stay on the 16x16-tile kernels
   int int4_gemm32_min_rows;  // 0 = default (256), else rows from which the 32x32-tile kernel takes over
   int row_tiles;           // 0 = heuristic, else 1/2/4 tiles of 16 activation rows per workgroup (both matmuls)
 };
@@ -61,6 +61,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, ui
 // prefetch pipeline once per use.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 #endif
+
+// many-row int8 matmul on 32x32 MFMA tiles (e2h_int8_gemm.hip); xsum: scratch for the sums of x, xsum_bytes large
+int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, float *xsum, int64_t xsum_bytes, int M,
+                int N, int K, hipStream_t stream);
 
 // streaming int8 matmul (e2h_int8_stream.hip)
 int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int M, int N, int K, void *workspace,

@@ -356,6 +356,17 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
     a.y = y + m0 * N;
     a.M = static_cast<int>(M - m0 < max_rows ? M - m0 : max_rows);
     int rc;
+    const int min32 = options().int4_gemm32_min_rows > 0 ? options().int4_gemm32_min_rows : 256;
+    if (mt == 4 && a.M >= min32 && !options().int4_no_gemm32 && workspace && static_cast<int64_t>(N) * K < (int64_t{1} << 32)) {
+      // many rows: 32x32-tile kernel; the sums of x go to the partial-tile area of the workspace (no K split here)
+      const int64_t avail = workspace_bytes - static_cast<int64_t>(kTicketBytes8);
+      const int64_t need = static_cast<int64_t>(K / 128) * (((a.M + 63) / 64) * 64) * 4;
+      if (need <= avail) {
+        rc = int8_gemm32(a.x, q, scales, a.y, reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + kTicketBytes8), avail, a.M, N, K, stream);
+        if (rc != E2H_OK) return rc;
+        continue;
+      }
+    }
     if (mt == 1) rc = t == 2 ? (wk == 2 ? launch8<1, 2, 4, 2>(a) : launch8<1, 2, 4, 1>(a)) : (wk == 2 ? launch8<1, 1, 4, 2>(a) : launch8<1, 1, 4, 1>(a));
     else if (mt == 2) rc = t == 2 ? (wk == 2 ? launch8<2, 2, 4, 2>(a) : launch8<2, 2, 4, 1>(a)) : (wk == 2 ? launch8<2, 1, 4, 2>(a) : launch8<2, 1, 4, 1>(a));
     else rc = t == 2 ? launch8<4, 2, 4, 1>(a) : launch8<4, 1, 4, 1>(a);
