@@ -45,7 +45,7 @@ struct Options {
   int int8_force_generic;  // 1 = always use the generic (bounds-checked) int8 kernel
   int int4_no_xsum;        // 1 = many-row int4 calls compute the group sums of x inside the matmul (no pre-pass)
   int int4_no_gemm32;      // 1 = many-row calls (int4 and int8) stay on the 16x16-tile kernels
-  int int4_gemm32_min_rows;  // 0 = default (256), else rows from which the 32x32-tile kernel takes over
+  int int4_gemm32_min_rows;  // 0 = by workgroup count, else rows from which the 32x32-tile kernels take over
   int row_tiles;           // 0 = heuristic, else 1/2/4 tiles of 16 activation rows per workgroup (both matmuls)
 };
 Options &options();

@@ -727,8 +727,11 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
         a.xsum = xs;
         a.xsum_stride = stride;
         // 32x32-tile kernel for whole 128-row blocks' worth of work
-        const int min32 = options().int4_gemm32_min_rows > 0 ? options().int4_gemm32_min_rows : 256;
-        if (a.M >= min32 && !options().int4_no_gemm32) {
+        // the 128 x 128-output workgroups of that kernel pay off once there are enough of them to fill the chip
+        // (measured crossover on the 7B shapes: about 320 workgroups)
+        const long long wgs32 = static_cast<long long>((a.M + 127) / 128) * ((a.N + 127) / 128);
+        const bool use32 = options().int4_gemm32_min_rows > 0 ? a.M >= options().int4_gemm32_min_rows : wgs32 >= 320;
+        if (use32 && !options().int4_no_gemm32) {
           const int rc32 = int4_gemm32(a.x, a.packed, a.sz, a.y, xs, stride, a.M, a.N, a.K, groupsize, a.stream);
           if (rc32 != E2H_OK) return rc32;
           continue;

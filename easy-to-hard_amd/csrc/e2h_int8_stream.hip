@@ -356,8 +356,9 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
     a.y = y + m0 * N;
     a.M = static_cast<int>(M - m0 < max_rows ? M - m0 : max_rows);
     int rc;
-    const int min32 = options().int4_gemm32_min_rows > 0 ? options().int4_gemm32_min_rows : 256;
-    if (mt == 4 && a.M >= min32 && !options().int4_no_gemm32 && workspace && static_cast<int64_t>(N) * K < (int64_t{1} << 32)) {
+    const long long wgs32 = static_cast<long long>((a.M + 127) / 128) * ((N + 127) / 128);
+    const bool use32 = options().int4_gemm32_min_rows > 0 ? a.M >= options().int4_gemm32_min_rows : wgs32 >= 320;
+    if (mt == 4 && use32 && !options().int4_no_gemm32 && workspace && static_cast<int64_t>(N) * K < (int64_t{1} << 32)) {
       // many rows: 32x32-tile kernel; the sums of x go to the partial-tile area of the workspace (no K split here)
       const int64_t avail = workspace_bytes - static_cast<int64_t>(kTicketBytes8);
       const int64_t need = static_cast<int64_t>(K / 128) * (((a.M + 63) / 64) * 64) * 4;
