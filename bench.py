@@ -46,6 +46,9 @@ def parse_args():
     ap.add_argument("--max-new", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--gemv-reps", type=int, default=20)
+    ap.add_argument("--reward", action="store_true",
+                    help="reward-model scoring workload instead of decode: one fully causal pass over --batch x --prompt "
+                         "tokens per step (use --mode int8 --batch 64 --prompt 768 for the reference's scoring configuration)")
     ap.add_argument("--per-shape", default="",
                     help="comma-separated row counts M: time every distinct quantized-linear shape of the model at each M "
                          "(all layers' instances back to back, so the weights rotate) and print one JSON line")
@@ -245,6 +248,43 @@ def measure_cpu_baseline(model, batch, groupsize):
     }
 
 
+def run_reward_scoring(args, cfg, dev):
+    """Scoring pass of a RewardModel (2-row head, mean over its rows): every linear sees batch * prompt rows, so the
+    quantized linears are MFMA-bound.  One step = one pass over the whole batch; value = scored tokens per second."""
+    import torch
+
+    from easy_to_hard_amd.generate import model_score
+    from easy_to_hard_amd.model import random_quantized_transformer
+
+    model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234, reward_head_rows=2)
+    batch, t = args.batch, args.prompt
+    ids = torch.randint(0, cfg.vocab_size, (batch, t), generator=torch.Generator().manual_seed(1234)).to(dev)
+    steps, warmup = min(args.steps, 8), min(args.warmup, 2)
+    for _ in range(max(warmup, 1)):
+        rewards = model_score(model, ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rewards = model_score(model, ids)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lins = quantized_linears(model)
+    flops = sum(2.0 * batch * t * m.out_features * m.in_features for _, m in lins)
+    print(json.dumps({
+        "metric": "reward-model scoring tokens/s (Llama-7B shape, weight-only quantized linears)",
+        "value": round(batch * t * steps / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(elapsed / steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"random-init Llama {args.model}-shaped reward model, {args.mode} weight-only linears, "
+                               f"fully causal scoring pass, batch {batch} x {t} tokens", "batch": batch, "tokens": t},
+        "roofline": {"bound": "mfma", "achieved": round(flops * steps / elapsed / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": round(flops * steps / elapsed / 1e12 / 2500.0, 4), "traffic": None,
+                     "note": "linear-layer flops over the whole step time (attention, norms and elementwise kernels included in the time)"},
+        "cpu_baseline": None,
+        "finite": bool(torch.isfinite(rewards.float()).all()),
+    }))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -264,6 +304,13 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     cfg = ModelArgs.from_name(args.model)
+    if args.reward:
+        if args.mode != "int8":
+            # the 2-row score head cannot be an int4 linear (out_features % 8 != 0 asserts, as in the reference)
+            print("bench.py --reward runs the int8 configuration only (use --mode int8)", file=sys.stderr)
+            sys.exit(2)
+        run_reward_scoring(args, cfg, dev)
+        return
     t0 = time.time()
     model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234)
     torch.cuda.synchronize()
