@@ -31,6 +31,7 @@ _SIGNATURES = {
     "e2h_rmsnorm": (c_int, [_P, _P, _P, c_int64, c_int64, c_float, _P]),
     "e2h_add_rmsnorm": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "e2h_rope_kv_write": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
+    "e2h_rope_kv_write_seq": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, _P]),
     "e2h_silu_mul": (c_int, [_P, _P, _P, c_int64, _P]),
     "e2h_int4_mm_rope_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, _P]),
     "e2h_sample_top_k": (c_int, [_P, c_int64, _P, _P, _P, c_int64, c_int64, c_float, c_int, _P]),

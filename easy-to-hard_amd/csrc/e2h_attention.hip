@@ -221,22 +221,29 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
 }
 
 // ------------------------------------------------------------------------------------------------
-// RoPE + KV write for one new token per sequence.  qkv [B, (H + 2 Hkv) * D] bf16 (rows ordered q | k | v),
-// freqs [S, D/2, 2] bf16 (cos, sin).  Writes q_out [B, H, D] (rotated) and the caches at input_pos.
-// Rotation of interleaved pairs in float32, rounded to bf16 (reference :400-412).
+// RoPE + KV write.  qkv [B * T, (H + 2 Hkv) * D] bf16 (row b * T + t, columns ordered q | k | v), T new tokens per
+// sequence at positions input_pos[0 .. T-1]; freqs [>= S, D/2, 2] bf16 (cos, sin).  Writes q_out [B, H, T, D]
+// (rotated, head-major as attention wants it) and k (rotated) / v into [B, Hkv, S, D] at the positions.
+// Rotation of interleaved pairs in float32, rounded to bf16 (reference :400-412); positions outside [0, S) write
+// nothing to the caches.  rows_by_token: k / v row = token index t instead of its position (a pass without KV
+// cache, where k and v are fresh tensors of exactly T rows).
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ freqs,
                                                             uint16_t *__restrict__ q_out, uint16_t *__restrict__ kc, uint16_t *__restrict__ vc,
-                                                            const int64_t *__restrict__ input_pos, int B, int H, int Hkv, int S, int D) {
+                                                            const int64_t *__restrict__ input_pos, int B, int T, int H, int Hkv, int S, int D, int rows_by_token) {
   const int pairs_per_row = (H + 2 * Hkv) * D / 2;
-  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= B * pairs_per_row) return;
-  const int b = idx / pairs_per_row, p = idx % pairs_per_row;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<int64_t>(B) * T * pairs_per_row) return;
+  const int row = static_cast<int>(idx / pairs_per_row), p = static_cast<int>(idx % pairs_per_row);
+  const int b = row / T, t = row % T;
   const int head = (2 * p) / D, dpair = p % (D / 2);
-  const int pos = static_cast<int>(input_pos[0]);
+  const int pos = static_cast<int>(input_pos[t]);   // rotation angle
+  const int slot = rows_by_token ? t : pos;         // row of the k / v tensors that receives this token
+  const bool pos_ok = pos >= 0 && slot >= 0 && slot < S;
   const uint32_t raw = reinterpret_cast<const uint32_t *>(qkv)[idx];
   const float x0 = __builtin_bit_cast(float, raw << 16), x1 = __builtin_bit_cast(float, raw & 0xFFFF0000u);
   if (head < H + Hkv) {
+    if (!pos_ok) return;  // no angle for such a position
     const uint32_t f = reinterpret_cast<const uint32_t *>(freqs)[static_cast<size_t>(pos) * (D / 2) + dpair];
     const float cs = __builtin_bit_cast(float, f << 16), sn = __builtin_bit_cast(float, f & 0xFFFF0000u);
     // two separately rounded products and their difference / sum, as torch evaluates the expression in float32
@@ -244,14 +251,14 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(const uint16_t *__re
     const float r1 = x1 * cs + x0 * sn;
     const uint32_t o = static_cast<uint32_t>(f32_to_bf16_rne(r0)) | (static_cast<uint32_t>(f32_to_bf16_rne(r1)) << 16);
     if (head < H) {
-      reinterpret_cast<uint32_t *>(q_out)[(static_cast<size_t>(b) * H + head) * (D / 2) + dpair] = o;
+      reinterpret_cast<uint32_t *>(q_out)[((static_cast<size_t>(b) * H + head) * T + t) * (D / 2) + dpair] = o;
     } else {
       const int hk = head - H;
-      reinterpret_cast<uint32_t *>(kc)[((static_cast<size_t>(b) * Hkv + hk) * S + pos) * (D / 2) + dpair] = o;
+      reinterpret_cast<uint32_t *>(kc)[((static_cast<size_t>(b) * Hkv + hk) * S + slot) * (D / 2) + dpair] = o;
     }
-  } else {
+  } else if (pos_ok) {
     const int hk = head - H - Hkv;
-    reinterpret_cast<uint32_t *>(vc)[((static_cast<size_t>(b) * Hkv + hk) * S + pos) * (D / 2) + dpair] = raw;
+    reinterpret_cast<uint32_t *>(vc)[((static_cast<size_t>(b) * Hkv + hk) * S + slot) * (D / 2) + dpair] = raw;
   }
 }
 
@@ -327,16 +334,26 @@ extern "C" int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const u
   return launch_status();
 }
 
+extern "C" int e2h_rope_kv_write_seq(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache,
+                                     const int64_t *input_pos, int64_t batch, int64_t seqlen, int64_t n_head, int64_t n_kv_head,
+                                     int64_t cache_len, int64_t head_dim, int rows_by_token, void *stream) {
+  if (!qkv || !freqs_cis || !q_out || !k_cache || !v_cache || !input_pos) return E2H_ERR_NULL_POINTER;
+  if (batch < 1 || seqlen < 1 || n_head < 1 || n_kv_head < 1 || head_dim < 2 || head_dim % 2 != 0 || cache_len < 1 || cache_len > INT32_MAX)
+    return E2H_ERR_BAD_SHAPE;
+  const int64_t pairs = batch * seqlen * (n_head + 2 * n_kv_head) * head_dim / 2;
+  if (batch * seqlen > INT32_MAX || (pairs + 255) / 256 > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(qkv) & 3u) || (reinterpret_cast<uintptr_t>(freqs_cis) & 3u) || (reinterpret_cast<uintptr_t>(q_out) & 3u) ||
+      (reinterpret_cast<uintptr_t>(k_cache) & 3u) || (reinterpret_cast<uintptr_t>(v_cache) & 3u) || (reinterpret_cast<uintptr_t>(input_pos) & 7u))
+    return E2H_ERR_MISALIGNED;
+  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), qkv,
+                     freqs_cis, q_out, k_cache, v_cache, input_pos, (int)batch, (int)seqlen, (int)n_head, (int)n_kv_head, (int)cache_len, (int)head_dim, rows_by_token ? 1 : 0);
+  return launch_status();
+}
+
 extern "C" int e2h_rope_kv_write(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache,
                                  const int64_t *input_pos, int64_t batch, int64_t n_head, int64_t n_kv_head, int64_t cache_len,
                                  int64_t head_dim, void *stream) {
-  if (!qkv || !freqs_cis || !q_out || !k_cache || !v_cache || !input_pos) return E2H_ERR_NULL_POINTER;
-  if (batch < 1 || n_head < 1 || n_kv_head < 1 || head_dim < 2 || head_dim % 2 != 0) return E2H_ERR_BAD_SHAPE;
-  const int64_t pairs = batch * (n_head + 2 * n_kv_head) * head_dim / 2;
-  if (pairs > INT32_MAX) return E2H_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), qkv,
-                     freqs_cis, q_out, k_cache, v_cache, input_pos, (int)batch, (int)n_head, (int)n_kv_head, (int)cache_len, (int)head_dim);
-  return launch_status();
+  return e2h_rope_kv_write_seq(qkv, freqs_cis, q_out, k_cache, v_cache, input_pos, batch, 1, n_head, n_kv_head, cache_len, head_dim, 0, stream);
 }
 
 extern "C" int e2h_silu_mul(const uint16_t *a, const uint16_t *b, uint16_t *y, int64_t n, void *stream) {

@@ -158,6 +158,15 @@ class Attention(nn.Module):
                 and self.freqs_table is not None and self.head_dim in (64, 128)
                 and (self.n_head // self.n_local_heads) in (1, 2, 4, 8))
 
+    def _can_fuse_prefill_rope(self, x: Tensor, input_pos: Optional[Tensor], fully_causal: bool) -> bool:
+        if not (_fusable(x) and self.freqs_table is not None and self.freqs_table.dtype == torch.bfloat16):
+            return False
+        if input_pos is None or input_pos.dtype != torch.int64 or input_pos.numel() != x.shape[1] or self.head_dim % 2:
+            return False
+        if fully_causal:
+            return True
+        return self.kv_cache is not None and self.freqs_table.shape[0] >= self.kv_cache.k_cache.shape[2]
+
     def forward(self, x: Tensor, freqs_cis: Optional[Tensor], mask: Optional[Tensor], input_pos: Optional[Tensor] = None,
                 fully_causal: bool = False) -> Tensor:
         bsz, seqlen, _ = x.shape
@@ -176,12 +185,25 @@ class Attention(nn.Module):
                                       self.n_head, self.n_local_heads, self.head_dim)
             y = ops.decode_attention(q, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, self.left_pad_mask_pos)
             return self.wo(y.view(bsz, 1, self.dim))
-        q, k, v = self.wqkv(x).split([self.dim, kv_size, kv_size], dim=-1)
-        q = apply_rotary_emb(q.view(bsz, seqlen, self.n_head, self.head_dim), freqs_cis).transpose(1, 2)
-        k = apply_rotary_emb(k.view(bsz, seqlen, self.n_local_heads, self.head_dim), freqs_cis).transpose(1, 2)
-        v = v.view(bsz, seqlen, self.n_local_heads, self.head_dim).transpose(1, 2)
-        if not fully_causal:
-            k, v = self.kv_cache.update(input_pos, k, v)
+        if self._can_fuse_prefill_rope(x, input_pos, fully_causal):
+            # many new tokens per sequence: rotation, head-major layout and cache write in one pass over qkv
+            qkv = self.wqkv(x)
+            if fully_causal:
+                # no cache: k and v of exactly this length, rows in token order; the angles are those of input_pos
+                k = torch.empty((bsz, self.n_local_heads, seqlen, self.head_dim), dtype=torch.bfloat16, device=x.device)
+                v = torch.empty_like(k)
+            else:
+                k, v = self.kv_cache.k_cache, self.kv_cache.v_cache
+            q = ops.rope_kv_write_seq(qkv, self.freqs_table, k, v, input_pos, self.n_head, self.n_local_heads, self.head_dim,
+                                      rows_by_token=fully_causal)
+            k, v = k[:bsz], v[:bsz]
+        else:
+            q, k, v = self.wqkv(x).split([self.dim, kv_size, kv_size], dim=-1)
+            q = apply_rotary_emb(q.view(bsz, seqlen, self.n_head, self.head_dim), freqs_cis).transpose(1, 2)
+            k = apply_rotary_emb(k.view(bsz, seqlen, self.n_local_heads, self.head_dim), freqs_cis).transpose(1, 2)
+            v = v.view(bsz, seqlen, self.n_local_heads, self.head_dim).transpose(1, 2)
+            if not fully_causal:
+                k, v = self.kv_cache.update(input_pos, k, v)
         rep = self.n_head // self.n_local_heads
         if rep > 1:
             k = k.repeat_interleave(rep, dim=1)

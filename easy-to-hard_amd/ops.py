@@ -398,6 +398,24 @@ def rope_kv_write(qkv, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head
     return q
 
 
+def rope_kv_write_seq(qkv, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head, head_dim, rows_by_token=False):
+    """qkv bf16 [B, T, (H + 2 Hkv) * D] -> rotated q [B, H, T, D]; rotated k and v are written into the caches
+    [>= B, Hkv, S, D] at rows input_pos [T] (int64 on the device), or at rows 0 .. T-1 with rows_by_token (no KV cache)."""
+    _need_gpu(qkv, freqs_cis, k_cache, v_cache, input_pos)
+    assert qkv.dtype == torch.bfloat16 and freqs_cis.dtype == torch.bfloat16 and input_pos.dtype == torch.int64 and qkv.dim() == 3
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and freqs_cis.is_contiguous()
+    qkv = qkv.contiguous()
+    bsz, t = qkv.shape[0], qkv.shape[1]
+    assert input_pos.numel() == t and qkv.shape[2] == (n_head + 2 * n_kv_head) * head_dim
+    assert k_cache.shape[0] >= bsz and k_cache.shape[1] == n_kv_head and k_cache.shape[3] == head_dim and v_cache.shape == k_cache.shape
+    assert rows_by_token or freqs_cis.shape[0] >= k_cache.shape[2]  # (with rows_by_token the positions must index freqs_cis)
+    q = torch.empty((bsz, n_head, t, head_dim), dtype=torch.bfloat16, device=qkv.device)
+    rc = _lib_for(qkv).e2h_rope_kv_write_seq(_ptr(qkv), _ptr(freqs_cis), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(input_pos.contiguous()),
+                                             bsz, t, n_head, n_kv_head, k_cache.shape[2], head_dim, 1 if rows_by_token else 0, _stream(qkv))
+    _lib.check(rc, "e2h_rope_kv_write_seq")
+    return q
+
+
 def int4_rope_kv_supported(x, wqkv, freqs_cis, k_cache):
     """True when the fused projection + RoPE + cache write covers (x [B, 1, K], a WeightOnlyInt4Linear)."""
     if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 64):

@@ -191,6 +191,16 @@ int e2h_rope_kv_write(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *
                       uint16_t *v_cache, const int64_t *input_pos, int64_t batch, int64_t n_head,
                       int64_t n_kv_head, int64_t cache_len, int64_t head_dim, void *stream);
 
+/* The same for seqlen new tokens per sequence (prefill, scoring): qkv [batch * seqlen, (n_head + 2 n_kv_head) * head_dim]
+ * with row b * seqlen + t, input_pos [seqlen] int64 on the device, q_out [batch, n_head, seqlen, head_dim] (head-major,
+ * as scaled_dot_product_attention takes it, reference :296 transposes to it); k (rotated) and v go to
+ * [batch, n_kv_head, cache_len, head_dim] at row input_pos[t], or at row t when rows_by_token != 0 (a pass without
+ * KV cache: fresh k / v tensors with cache_len = seqlen; the rotation still uses input_pos[t]).  Rows outside
+ * [0, cache_len) are not written. */
+int e2h_rope_kv_write_seq(const uint16_t *qkv, const uint16_t *freqs_cis, uint16_t *q_out, uint16_t *k_cache,
+                          uint16_t *v_cache, const int64_t *input_pos, int64_t batch, int64_t seqlen, int64_t n_head,
+                          int64_t n_kv_head, int64_t cache_len, int64_t head_dim, int rows_by_token, void *stream);
+
 /* F.silu(a) * b with bf16 rounding after each op (reference FeedForward.forward :359-360). n elements, n % 8 == 0. */
 int e2h_silu_mul(const uint16_t *a, const uint16_t *b, uint16_t *y, int64_t n, void *stream);
 

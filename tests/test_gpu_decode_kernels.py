@@ -112,3 +112,52 @@ def test_fused_decode_step_matches_stock_decode_step():
             model_mod.FUSED_DECODE = True
     err = (logits[True] - logits[False]).abs().max() / logits[False].abs().max()
     assert err < 2e-2, err
+
+
+@pytest.mark.parametrize("n_head,n_kv,d", [(4, 4, 64), (8, 2, 128)])
+@pytest.mark.parametrize("by_token", [False, True])
+def test_rope_kv_write_seq_matches_stock_ops(n_head, n_kv, d, by_token):
+    """Many tokens per sequence: q comes back head-major and rotated, k / v land in the cache rows of their positions
+    (or in token order for a cache-less pass) with exactly the bits of apply_rotary_emb + KVCache.update."""
+    bsz, t, s_max = 2, 7, 24
+    gen = torch.Generator().manual_seed(n_head * 3 + d)
+    qkv = torch.randn((bsz, t, (n_head + 2 * n_kv) * d), generator=gen).to(torch.bfloat16).to(DEV)
+    freqs = precompute_freqs_cis(s_max, d, 10000, device=DEV)
+    input_pos = torch.arange(5, 5 + t, device=DEV)
+    rows = t if by_token else s_max
+    kc0 = torch.randn((bsz + 1, n_kv, rows, d), generator=gen).to(torch.bfloat16).to(DEV)
+    vc0 = torch.randn((bsz + 1, n_kv, rows, d), generator=gen).to(torch.bfloat16).to(DEV)
+    kc, vc = kc0.clone(), vc0.clone()
+    q_out = ops.rope_kv_write_seq(qkv, freqs, kc, vc, input_pos, n_head, n_kv, d, rows_by_token=by_token)
+    q, k, v = qkv.split([n_head * d, n_kv * d, n_kv * d], dim=-1)
+    fc = freqs[input_pos]
+    q_ref = apply_rotary_emb(q.view(bsz, t, n_head, d), fc).transpose(1, 2)
+    k_ref = apply_rotary_emb(k.view(bsz, t, n_kv, d), fc).transpose(1, 2)
+    v_ref = v.view(bsz, t, n_kv, d).transpose(1, 2)
+    assert q_out.shape == (bsz, n_head, t, d) and torch.equal(q_out, q_ref)
+    kc_ref, vc_ref = kc0.clone(), vc0.clone()
+    dest = torch.arange(t, device=DEV) if by_token else input_pos
+    kc_ref[:bsz].index_copy_(2, dest, k_ref)
+    vc_ref[:bsz].index_copy_(2, dest, v_ref)
+    assert torch.equal(kc, kc_ref) and torch.equal(vc, vc_ref)
+
+
+@pytest.mark.parametrize("fully_causal", [False, True])
+def test_fused_prefill_matches_stock_prefill(fully_causal):
+    model = Transformer.from_name("tiny-gqa-test")
+    init_random_(model, seed=6, std=0.05)
+    model = model.to(device=DEV, dtype=torch.bfloat16).eval()
+    bsz, t = 3, 11
+    ids = torch.randint(0, 512, (bsz, t), generator=torch.Generator().manual_seed(4)).to(DEV)
+    out = {}
+    for fused in (False, True):
+        model_mod.FUSED_DECODE = fused
+        try:
+            model.max_seq_length = -1
+            model.setup_caches(bsz, 32, kv_cache=not fully_causal)
+            with torch.no_grad():
+                out[fused] = model(ids, torch.arange(0, t, device=DEV), fully_causal=fully_causal).float()
+        finally:
+            model_mod.FUSED_DECODE = True
+    err = (out[True] - out[False]).abs().max() / out[False].abs().max()
+    assert err < 2e-2, err
