@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *_
   const int b = blockIdx.x / Hkv, hk = blockIdx.x % Hkv;
   const int pos = static_cast<int>(input_pos[0]);
   const int first = left_pad ? static_cast<int>(left_pad[b]) : 0;
-  const int n_live = pos + 1;
+  const int n_live = pos + 1 < S ? pos + 1 : S;  // never past the cache, whatever the position tensor holds
 
   float qf[REP][8];
 #pragma unroll

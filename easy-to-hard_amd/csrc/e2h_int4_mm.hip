@@ -573,8 +573,7 @@ int launch(const LaunchArgs &a) {
 struct Shape {
   int t, wn, wk;
 };
-constexpr Shape kShapes[] = {{1, 4, 1}, {1, 4, 2}, {1, 4, 4}, {1, 3, 4}, {1, 2, 4}, {1, 2, 2}, {1, 1, 4},
-                             {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {2, 3, 2}, {4, 4, 1}};
+constexpr Shape kShapes[] = {{1, 4, 1}, {1, 4, 2}, {1, 2, 2}, {2, 4, 1}, {2, 4, 2}, {2, 2, 2}, {4, 4, 1}};
 
 template <int G, int IKT>
 int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
@@ -584,8 +583,8 @@ int dispatch_shape(int mt, Shape sh, const LaunchArgs &a) {
     if (mt == 1) return launch<G, IKT, 1, TV, WNV, WKV>(a);                     \
     if (mt == 2) return launch<G, IKT, 2, TV, WNV, WKV>(a);                     \
   }
-    E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 4, 4) E2H_CASE(1, 3, 4) E2H_CASE(1, 2, 4) E2H_CASE(1, 2, 2)
-    E2H_CASE(1, 1, 4) E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(2, 3, 2) E2H_CASE(4, 4, 1)
+    E2H_CASE(1, 4, 1) E2H_CASE(1, 4, 2) E2H_CASE(1, 2, 2)
+    E2H_CASE(2, 4, 1) E2H_CASE(2, 4, 2) E2H_CASE(2, 2, 2) E2H_CASE(4, 4, 1)
 #undef E2H_CASE
     if (a.xsum) {
       if (sh.t == 2) return launch<G, IKT, 4, 2, 4, 1, kPlain, true>(a);
@@ -682,9 +681,8 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     // many rows of x (prefill, scoring): every weight fragment feeds four row tiles straight from registers;
     // wide column blocks keep the LDS traffic for activation fragments below the MFMA rate
     const int opt_t4 = options().int4_rows_per_wave / 16;
-    const long long wgs4 = static_cast<long long>((tiles16 + 15) / 16) * m_chunks;
-    (void)wgs4;
-    sh = Shape{opt_t4 ? opt_t4 : (static_cast<long long>((tiles16 + 7) / 8) * m_chunks >= kCUs ? 2 : 1), 4, 1};  // T = 2 measured best (830 TFLOP/s at M = 8192)
+    // two weight tiles per wave once that still leaves a workgroup per CU (measured best of T = 1 / 2 / 4)
+    sh = Shape{opt_t4 ? opt_t4 : (static_cast<long long>((tiles16 + 7) / 8) * m_chunks >= kCUs ? 2 : 1), 4, 1};
   }
   const int opt_t = options().int4_rows_per_wave / 16, opt_wk = options().int4_k_groups, opt_wn = options().int4_col_waves;
   if (wide_ok && mt <= 2 && (opt_t || opt_wk || opt_wn)) {
@@ -757,7 +755,10 @@ template <int G>
 int dispatch_gate(int mt, int wn, const LaunchArgs &a) {
 #define E2H_GATE_CASE(MTV, WNV) \
   if (mt == MTV && wn == WNV) return launch<G, 8, MTV, 2, WNV, 2, kGate>(a);
-  E2H_GATE_CASE(1, 4) E2H_GATE_CASE(2, 4) E2H_GATE_CASE(1, 3) E2H_GATE_CASE(2, 3) E2H_GATE_CASE(1, 2) E2H_GATE_CASE(2, 2)
+  E2H_GATE_CASE(1, 4) E2H_GATE_CASE(2, 4) E2H_GATE_CASE(1, 2) E2H_GATE_CASE(2, 2)
+  if constexpr (G == 128) {  // three column waves only where the registers suffice
+    E2H_GATE_CASE(1, 3) E2H_GATE_CASE(2, 3)
+  }
 #undef E2H_GATE_CASE
   return E2H_ERR_BAD_SHAPE;
 }
