@@ -181,3 +181,55 @@ def test_model_shapes_match_reference_configs():
         t = Transformer(b)
     assert t.layers[0].attention.wqkv.weight.shape == (10240, 8192)
     assert ModelArgs.from_name("llemma-7b").block_size == 4096
+
+
+def test_fused_and_sampling_entry_points_validate_arguments():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)  # never dereferenced: validation fails first
+    null = ctypes.c_void_p(0)
+    # gated launch: at most 64 rows, inner_k_tiles 8 only, group size 32 / 64 / 128
+    assert lib.e2h_int4_mm_silu_gate(p, p, p, p, p, p, 65, 64, 128, 128, 8, None) == -2
+    assert lib.e2h_int4_mm_silu_gate(p, p, p, p, p, p, 32, 64, 128, 128, 4, None) == -4
+    assert lib.e2h_int4_mm_silu_gate(p, p, p, p, p, p, 32, 64, 256, 256, 8, None) == -3
+    assert lib.e2h_int4_mm_silu_gate(p, null, p, p, p, p, 32, 64, 128, 128, 8, None) == -1
+    # projection + RoPE + cache write: odd head_dim, too many sequences, K not in whole chunks
+    assert lib.e2h_int4_mm_rope_kv(p, p, p, p, p, p, p, p, 4, 2, 2, 63, 16, 128, 128, 8, None) == -2
+    assert lib.e2h_int4_mm_rope_kv(p, p, p, p, p, p, p, p, 65, 2, 2, 64, 16, 128, 128, 8, None) == -2
+    assert lib.e2h_int4_mm_rope_kv(p, p, p, p, p, p, p, p, 4, 2, 2, 64, 16, 192, 64, 8, None) == -4
+    assert lib.e2h_rope_kv_write_seq(p, p, p, p, p, p, 2, 0, 2, 2, 16, 64, 0, None) == -2
+    assert lib.e2h_rope_kv_write_seq(p, p, p, p, p, null, 2, 3, 2, 2, 16, 64, 0, None) == -1
+    # sampling: row stride shorter than the vocabulary, negative top_k, misaligned q
+    assert lib.e2h_sample_top_k(p, 10, p, p, p, 2, 16, 1.0, 0, None) == -2
+    assert lib.e2h_sample_top_k(p, 16, p, p, p, 2, 16, 1.0, -1, None) == -2
+    assert lib.e2h_sample_top_k(p, 16, ctypes.c_void_p(4098), p, p, 2, 16, 1.0, 0, None) == -5
+    for name in (b"row_tiles", b"int4_no_xsum", b"int4_no_gemm32", b"int4_gemm32_min_rows"):
+        assert lib.e2h_set_option(name, 0) == 0
+    assert lib.e2h_set_option(b"row_tiles", 3) == -8
+
+
+def test_sampling_host_path_on_cpu_tensors():
+    """generate.sample falls back to the reference's op chain for inputs the kernel does not take (CPU, float32)."""
+    import torch
+
+    from easy_to_hard_amd.generate import logits_to_probs, multinomial_sample_one_no_sync, sample
+
+    torch.manual_seed(0)
+    logits = torch.randn(3, 2, 50)
+    probs = logits_to_probs(logits[:, -1], temperature=0.7, top_k=5)
+    assert probs.shape == (3, 50) and torch.allclose(probs.sum(-1), torch.ones(3))
+    assert torch.all((probs > 0).sum(-1) == 5)
+    idx = multinomial_sample_one_no_sync(probs)
+    assert idx.shape == (3, 1) and idx.dtype == torch.int and torch.all(probs.gather(1, idx.long()) > 0)
+    idx2, probs2 = sample(logits, temperature=0.7, top_k=5)
+    assert torch.allclose(probs2, probs) and idx2.shape == (3, 1)
+    # temperature -> 0 is clamped at 1e-5 and degenerates to arg-max
+    idx3, _ = sample(logits, temperature=0.0, top_k=None)
+    assert torch.equal(idx3[:, 0].long(), logits[:, -1].argmax(-1))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert proc.returncode == 2 and "one GPU" in proc.stderr
