@@ -9,11 +9,14 @@
 //   acc0[m,n] = -128 * sum_k x[m,k],
 // built before the main loop from per-128 sums of x (a one-pass pre-kernel) with v_mfma_f32_32x32x2_f32.
 //
-// Main loop, v_mfma_f32_32x32x16_bf16: lane L = 32*h + n supplies weight row n0 + n; per 32-wide k span t it loads
-// the 16 bytes k = 32 t + 16 h .. +15 (one 128-bit load), bytes 0..7 feeding step (t, 0) and bytes 8..15 step
-// (t, 1).  The activation fragment of lane (h, m) for step (t, a) is then the 16 contiguous bytes
-// x[m][32 t + 16 h + 8 a .. +7]: staging into LDS is a plain 16-byte copy per piece.  A workgroup of 4 waves owns
-// 128 rows x 128 columns, each wave 2 x 2 tiles accumulating straight into its 64 accumulator registers (no
+// Main loop, v_mfma_f32_32x32x16_bf16: lane L = 32*h + n supplies weight row n0 + n; per 32-wide k span t its B
+// operands are the 16 bytes k = 32 t + 16 h .. +15, bytes 0..7 feeding step (t, 0) and bytes 8..15 step (t, 1).  The
+// activation fragment of lane (h, m) for step (t, a) is then the 16 contiguous bytes x[m][32 t + 16 h + 8 a .. +7].
+// Both operands are staged per 128-wide k chunk into LDS in fragment order by plain 16-byte copies (double buffered,
+// one LDS barrier per chunk): read straight from memory, a weight fragment would touch 32 different rows per load
+// instruction, and that address traffic -- not the arithmetic -- bounded an earlier form of this kernel (measured:
+// 38 % of its time).  Staged, every global load covers whole 128-byte rows.  A workgroup of WR x WC waves owns
+// 64 WR rows x 64 WC columns, each wave 2 x 2 tiles accumulating straight into its 64 accumulator registers (no
 // per-group scale to apply); workgroups are laid out over the XCDs as in the int4 kernel of the same shape.
 #include "e2h_common.h"
 #include "e2h_int4_unpack.h"
@@ -25,8 +28,7 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kChunkK8 = 128;
 constexpr int kFragB8 = 1024 + 32;
-constexpr int kStageB8 = 4 * 8 * kFragB8;
-constexpr int kRT8 = 2, kCT8 = 2;
+constexpr int kRT8 = 2, kCT8 = 2;  // 32x32 tiles per wave: rows x columns
 
 // four codes (one dword, already offset to unsigned) -> two dwords of bfloat16 pairs
 __device__ __forceinline__ void bytes4_to_bf16(uint32_t t, uint32_t &lo, uint32_t &hi) {
@@ -37,11 +39,22 @@ __device__ __forceinline__ void bytes4_to_bf16(uint32_t t, uint32_t &lo, uint32_
   hi = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
 }
 
-__global__ __launch_bounds__(256) void int8_gemm32_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
-                                                          const uint16_t *__restrict__ scales, uint16_t *__restrict__ y,
-                                                          const float *__restrict__ xsum, int xsum_stride, int M, int N, int K,
-                                                          int n_col_blocks, int cbx) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageB8];
+template <int WR, int WC>
+__global__ __launch_bounds__(64 * WR * WC) void int8_gemm32_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
+                                                                   const uint16_t *__restrict__ scales, uint16_t *__restrict__ y,
+                                                                   const float *__restrict__ xsum, int xsum_stride, int M, int N, int K,
+                                                                   int n_col_blocks, int cbx) {
+  constexpr int kThreads = 64 * WR * WC;
+  constexpr int kRows = 64 * WR, kCols = 64 * WC;
+  constexpr int kStageX = (2 * WR) * 8 * kFragB8;     // kRows x 128 k of activations, 8 fragments per 32-row tile
+  constexpr int kStageW = (2 * WC) * 4 * kFragB8;     // kCols x 128 k of weights, 4 fragments per 32-column tile
+  constexpr int kXRowsPerPass = kThreads / 16;        // 16 pieces of 16 bytes per activation row
+  constexpr int kXPieces = kRows / kXRowsPerPass;
+  constexpr int kWColsPerPass = kThreads / 8;         // 8 pieces of 16 bytes per weight row
+  constexpr int kWPieces = kCols / kWColsPerPass;
+  static_assert(kXRowsPerPass % 32 == 0 && kWColsPerPass % 32 == 0, "staging passes cover whole 32-wide tiles");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * (kStageX + kStageW)];
+  uint8_t *const lds_w = lds + 2 * kStageX;
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
@@ -52,23 +65,15 @@ __global__ __launch_bounds__(256) void int8_gemm32_kernel(const uint16_t *__rest
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wr = wave >> 1, wc = wave & 1;
+  const int wr = wave / WC, wc = wave % WC;
   const int n = lane & 31, h = lane >> 5;
-  const int row0 = rb * 128 + wr * 64;
-  const int col0 = cb * 128 + wc * 64;
+  const int row0 = rb * kRows + wr * 64;
+  const int col0 = cb * kCols + wc * 64;
   const int nchunks = K / kChunkK8;
 
   const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(q, static_cast<uint32_t>(static_cast<size_t>(N) * K));
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
   const __amdgpu_buffer_rsrc_t xs_rsrc = make_rsrc(xsum, static_cast<uint32_t>(static_cast<size_t>(nchunks) * xsum_stride * 4));
-
-  uint32_t wlane[kCT8];
-#pragma unroll
-  for (int ct = 0; ct < kCT8; ++ct) {
-    int col = col0 + 32 * ct + n;
-    col = col < N ? col : N - 1;
-    wlane[ct] = static_cast<uint32_t>(static_cast<size_t>(col) * K + 16 * h);
-  }
 
   // ---- accumulators start at -128 * sum_k x[m,k] (float32 MFMAs over the per-chunk sums of x) ------------------
   f32x16_t acc[kCT8][kRT8];
@@ -95,55 +100,66 @@ __global__ __launch_bounds__(256) void int8_gemm32_kernel(const uint16_t *__rest
     }
   }
 
-  // ---- activation staging: piece (row, w): k = 8 w .. 8 w + 7 = 32 t + 16 h + 8 a with w = 4 t + 2 h + a -------------
-  const int r0 = tid >> 4, within = tid & 15;
-  uint32_t xsrc[8];
+  // ---- staging.  Activations: piece (row, w), k = 8 w .. 8 w + 7 = 32 t + 16 h + 8 a with w = 4 t + 2 h + a, goes to
+  // fragment (row tile, step 2 t + a), lane (h, row % 32).  Weights: piece (col, pc), bytes 16 pc .. 16 pc + 15 =
+  // 32 t + 16 h with pc = 2 t + h, goes to fragment (column tile, t), lane (h, col % 32).
+  const int xr0 = tid >> 4, xw = tid & 15;
+  uint32_t xsrc[kXPieces];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int row = rb * 128 + r0 + 16 * i;
+  for (int i = 0; i < kXPieces; ++i) {
+    int row = rb * kRows + xr0 + kXRowsPerPass * i;
     row = row < M ? row : M - 1;
-    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + within * 8) * 2);
+    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + xw * 8) * 2);
   }
-  const int xdst0 = (2 * (within >> 2) + (within & 1)) * kFragB8 + (((within >> 1) & 1) * 32 + r0) * 16;
-  auto load_x = [&](u32x4_t (&r)[8], int ci) {
+  const int xdst0 = ((xr0 >> 5) * 8 + 2 * (xw >> 2) + (xw & 1)) * kFragB8 + (((xw >> 1) & 1) * 32 + (xr0 & 31)) * 16;
+  const int wc0 = tid >> 3, wpc = tid & 7;
+  uint32_t wsrc[kWPieces];
+#pragma unroll
+  for (int i = 0; i < kWPieces; ++i) {
+    int col = cb * kCols + wc0 + kWColsPerPass * i;
+    col = col < N ? col : N - 1;
+    wsrc[i] = static_cast<uint32_t>(static_cast<size_t>(col) * K + wpc * 16);
+  }
+  const int wdst0 = ((wc0 >> 5) * 4 + (wpc >> 1)) * kFragB8 + ((wpc & 1) * 32 + (wc0 & 31)) * 16;
+
+  struct Staged {
+    u32x4_t x[kXPieces], w[kWPieces];
+  };
+  auto load_next = [&](Staged &r, int ci) {
     const int cc = ci < nchunks ? ci : nchunks - 1;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(cc) * (kChunkK8 * 2), 0);
-  };
-  auto store_x = [&](const u32x4_t (&r)[8], int parity) {
-    uint8_t *buf = lds + (parity & 1) * kStageB8 + xdst0;
+    for (int i = 0; i < kXPieces; ++i) r.x[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(cc) * (kChunkK8 * 2), 0);
 #pragma unroll
-    for (int i = 0; i < 8; ++i)  // row = r0 + 16 i: row tile i / 2, row within the tile r0 + 16 (i % 2)
-      *reinterpret_cast<u32x4_t *>(buf + (i >> 1) * (8 * kFragB8) + (i & 1) * (16 * 16)) = r[i];
+    for (int i = 0; i < kWPieces; ++i) r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wsrc[i], static_cast<uint32_t>(cc) * kChunkK8, 0);
+  };
+  auto store_next = [&](const Staged &r, int parity) {
+    uint8_t *bx = lds + (parity & 1) * kStageX + xdst0;
+#pragma unroll
+    for (int i = 0; i < kXPieces; ++i) *reinterpret_cast<u32x4_t *>(bx + i * (kXRowsPerPass / 32) * (8 * kFragB8)) = r.x[i];
+    uint8_t *bw = lds_w + (parity & 1) * kStageW + wdst0;
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i) *reinterpret_cast<u32x4_t *>(bw + i * (kWColsPerPass / 32) * (4 * kFragB8)) = r.w[i];
   };
 
-  struct WRegs {
-    u32x4_t w[kCT8][4];
-  };
-  auto load_w = [&](WRegs &r, int ci) {
-    const int cc = ci < nchunks ? ci : nchunks - 1;
-#pragma unroll
-    for (int ct = 0; ct < kCT8; ++ct)
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-        r.w[ct][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[ct], static_cast<uint32_t>(cc) * kChunkK8 + 32u * t, 0);
-  };
-
-  auto compute = [&](const WRegs &r, int parity) {
-    const uint8_t *buf = lds + (parity & 1) * kStageB8 + (wr * kRT8) * (8 * kFragB8) + lane * 16;
+  auto compute = [&](int parity) {
+    const uint8_t *bx = lds + (parity & 1) * kStageX + (wr * kRT8) * (8 * kFragB8) + lane * 16;
+    const uint8_t *bw = lds_w + (parity & 1) * kStageW + (wc * kCT8) * (4 * kFragB8) + lane * 16;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
+      u32x4_t wq[kCT8];
+#pragma unroll
+      for (int ct = 0; ct < kCT8; ++ct) wq[ct] = *reinterpret_cast<const u32x4_t *>(bw + (ct * 4 + t) * kFragB8);
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
         const int s = 2 * t + a;
         bf16x8_t af[kRT8];
 #pragma unroll
-        for (int rt = 0; rt < kRT8; ++rt) af[rt] = *reinterpret_cast<const bf16x8_t *>(buf + (rt * 8 + s) * kFragB8);
+        for (int rt = 0; rt < kRT8; ++rt) af[rt] = *reinterpret_cast<const bf16x8_t *>(bx + (rt * 8 + s) * kFragB8);
 #pragma unroll
         for (int ct = 0; ct < kCT8; ++ct) {
           uint32_t u0, u1, u2, u3;
-          bytes4_to_bf16(r.w[ct][t][2 * a] ^ 0x80808080u, u0, u1);
-          bytes4_to_bf16(r.w[ct][t][2 * a + 1] ^ 0x80808080u, u2, u3);
+          bytes4_to_bf16(wq[ct][2 * a] ^ 0x80808080u, u0, u1);
+          bytes4_to_bf16(wq[ct][2 * a + 1] ^ 0x80808080u, u2, u3);
           const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, u32x4_t{u0, u1, u2, u3});
 #pragma unroll
           for (int rt = 0; rt < kRT8; ++rt) acc[ct][rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[rt], wf, acc[ct][rt], 0, 0, 0);
@@ -152,23 +168,14 @@ __global__ __launch_bounds__(256) void int8_gemm32_kernel(const uint16_t *__rest
     }
   };
 
-  WRegs ring[2];
-  u32x4_t xst[8];
-  load_x(xst, 0);
-  load_w(ring[0], 0);
-  store_x(xst, 0);
+  Staged st;
+  load_next(st, 0);
+  store_next(st, 0);
   lds_barrier();
-  for (int ci = 0; ci < nchunks; ci += 2) {
-    load_x(xst, ci + 1);
-    load_w(ring[1], ci + 1);
-    compute(ring[0], 0);
-    store_x(xst, 1);
-    lds_barrier();
-    if (ci + 1 >= nchunks) break;  // uniform
-    load_x(xst, ci + 2);
-    load_w(ring[0], ci + 2);
-    compute(ring[1], 1);
-    store_x(xst, 0);
+  for (int ci = 0; ci < nchunks; ++ci) {
+    load_next(st, ci + 1);       // in flight during the arithmetic of this chunk
+    compute(ci);
+    store_next(st, ci + 1);      // the other stage: everybody left it at the previous barrier
     lds_barrier();
   }
 
@@ -196,12 +203,13 @@ int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint
   if (static_cast<int64_t>(K / kChunkK8) * stride * 4 > xsum_bytes) return E2H_ERR_BAD_SHAPE;
   const int rc = launch_x_group_sums(x, xsum, M, K, stride, 128, stream);
   if (rc != E2H_OK) return rc;
-  const int n_col_blocks = (N + 127) / 128, n_row_blocks = (M + 127) / 128;
+  constexpr int WR = 2, WC = 4;  // 128 rows x 256 columns per workgroup of 8 waves, one workgroup per CU (135 KB of LDS)
+  const int n_col_blocks = (N + 64 * WC - 1) / (64 * WC), n_row_blocks = (M + 64 * WR - 1) / (64 * WR);
   const int cbx = (n_col_blocks + 7) / 8;
   const long long wgs = 8LL * cbx * n_row_blocks;
   if (wgs > 0x7FFFFFFFLL) return E2H_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(int8_gemm32_kernel, dim3(static_cast<unsigned>(wgs)), dim3(256), 0, stream, x, q, scales, y, xsum, stride, M, N, K,
-                     n_col_blocks, cbx);
+  hipLaunchKernelGGL((int8_gemm32_kernel<WR, WC>), dim3(static_cast<unsigned>(wgs)), dim3(64 * WR * WC), 0, stream, x, q, scales, y, xsum,
+                     stride, M, N, K, n_col_blocks, cbx);
   return launch_status();
 }
 
