@@ -14,9 +14,10 @@
 // k0 + {2j, 2j+1, 2j+8, 2j+9, 2j+16, ...} (j = 0..3); the lane loads the words with j = h (first 16-byte load)
 // and j = 2 + h (second), four 32-wide k spans p each.  Step (p, jp) multiplies the words (j = 2 jp + h, p) with
 // the activation fragment gathered in the same k order, so weights are never shuffled: one word is one B operand.
-// A workgroup of 4 waves owns 128 rows x 128 columns (each wave 64 x 64 = 2 x 2 tiles, 64 accumulator registers);
-// activations are staged per 128-wide k chunk into LDS in fragment order (double buffered, one LDS barrier per
-// chunk); every A fragment read feeds two column tiles and every unpacked word two row tiles.
+// A workgroup of WR x WC waves owns 64 WR rows x 64 WC columns (each wave 64 x 64 = 2 x 2 tiles, 64 accumulator
+// registers).  Activations and packed weights are both staged per 128-wide k chunk into LDS in fragment order (double
+// buffered, one LDS barrier per chunk): the global loads then cover whole contiguous 512-byte weight blocks and whole
+// activation rows, every A fragment read feeds two column tiles and every unpacked word two row tiles.
 //
 // Workgroup -> tile mapping: workgroup w runs on XCD w % 8; each XCD owns the column blocks cb = xcd (mod 8) and
 // walks them for one row block before moving to the next, so its L2 keeps that slice of the weights.
@@ -30,17 +31,26 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kChunkK = 128;
 constexpr int kFragB = 1024 + 32;                   // one 32-row x 16-k A fragment block in LDS (64 lanes x 16 B) + skew
-constexpr int kStageB = 4 * 8 * kFragB;             // 128 rows x 128 k
 constexpr int kRT = 2, kCT = 2;                     // 32x32 tiles per wave: rows x columns
 
-template <int G>
-__global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp,
-                                                          const uint32_t *__restrict__ sz, uint16_t *__restrict__ y,
-                                                          const float *__restrict__ xsum, int xsum_stride, int M, int N, int K,
-                                                          int n_col_blocks, int cbx) {
+template <int G, int WR, int WC>
+__global__ __launch_bounds__(64 * WR * WC) void int4_gemm32_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp,
+                                                                   const uint32_t *__restrict__ sz, uint16_t *__restrict__ y,
+                                                                   const float *__restrict__ xsum, int xsum_stride, int M, int N, int K,
+                                                                   int n_col_blocks, int cbx) {
   constexpr int NGRP = kChunkK / G;   // groups per chunk
   constexpr int SPG = G / 16;         // MFMA steps per group
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageB];
+  constexpr int kThreads = 64 * WR * WC;
+  constexpr int kRows = 64 * WR, kCols = 64 * WC;
+  constexpr int kStageX = (2 * WR) * 8 * kFragB;      // kRows x 128 k of activations, 8 fragments per 32-row tile
+  constexpr int kStageW = (2 * WC) * 2 * kFragB;      // kCols x 128 k of packed weights, 2 fragments (j pairs) per 32-column tile
+  constexpr int kXRowsPerPass = kThreads / 16;        // 16 pieces of 16 bytes per activation row
+  constexpr int kXPieces = kRows / kXRowsPerPass;
+  constexpr int kWTilesPerPass = kThreads / 32;       // 32 pieces of 16 bytes per 8-column weight block
+  constexpr int kWPieces = (kCols / 8) / kWTilesPerPass;
+  static_assert(kXRowsPerPass % 32 == 0 && kWTilesPerPass % 4 == 0, "staging passes cover whole 32-wide tiles");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * (kStageX + kStageW)];
+  uint8_t *const lds_w = lds + 2 * kStageX;
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
@@ -51,10 +61,10 @@ __global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__rest
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wr = wave >> 1, wc = wave & 1;
+  const int wr = wave / WC, wc = wave % WC;
   const int n = lane & 31, h = lane >> 5;
-  const int row0 = rb * 128 + wr * 64;
-  const int col0 = cb * 128 + wc * 64;
+  const int row0 = rb * kRows + wr * 64;
+  const int col0 = cb * kCols + wc * 64;
   const int KT = K / kChunkK;
   const int nchunks = K / kChunkK;
   const int ngroups = K / G;
@@ -64,18 +74,12 @@ __global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__rest
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
   const __amdgpu_buffer_rsrc_t xs_rsrc = make_rsrc(xsum, static_cast<uint32_t>(static_cast<size_t>(ngroups) * xsum_stride * 4));
 
-  // per-lane constant byte offsets
-  uint32_t wlane[kCT][2], szlane[kCT];
+  uint32_t szlane[kCT];  // byte offset of this lane's column inside one [N] row of (scale, zero) pairs
 #pragma unroll
   for (int ct = 0; ct < kCT; ++ct) {
     int col = col0 + 32 * ct + n;
     col = col < N ? col : N - 1;
     szlane[ct] = static_cast<uint32_t>(col) * 4u;
-#pragma unroll
-    for (int ld = 0; ld < 2; ++ld) {
-      const int j = 2 * ld + h;
-      wlane[ct][ld] = static_cast<uint32_t>((static_cast<size_t>(col >> 3) * KT * 32 + ((col & 7) * 4 + j)) * 16);
-    }
   }
 
   // ---- accumulators start as the zero-point term: sum_g X[m,g] * (z - 136 s)[g,n] in float32 MFMAs --------
@@ -112,54 +116,69 @@ __global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__rest
     }
   }
 
-  // ---- activation staging: 2048 16-byte pieces per chunk, 8 per thread ------------------------------
-  // piece (row, within): span p = within / 4 of 32 k, quarter u = within % 4; its dword e belongs to the fragment
-  // of step (p, e / 2), lane (h = e % 2, row % 32), register u.
-  const int r0 = tid >> 4, within = tid & 15;
-  uint32_t xsrc[8];
+  // ---- staging.  Activations: piece (row, within): span p = within / 4 of 32 k, quarter u = within % 4; its dword e
+  // belongs to the fragment of step (p, e / 2), lane (h = e % 2, row % 32), register u.  Weights: piece (8-column block,
+  // t) of a 512-byte block = the four words (column 8 blk + t / 4, j = t % 4): fragment (column tile, j / 2), lane
+  // (h = j % 2, column % 32).
+  const int xr0 = tid >> 4, xw = tid & 15;
+  uint32_t xsrc[kXPieces];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int row = rb * 128 + r0 + 16 * i;
+  for (int i = 0; i < kXPieces; ++i) {
+    int row = rb * kRows + xr0 + kXRowsPerPass * i;
     row = row < M ? row : M - 1;
-    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + within * 8) * 2);
+    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + xw * 8) * 2);
   }
-  const int xdst0 = (2 * (within >> 2)) * kFragB + r0 * 16 + (within & 3) * 4;
-  auto load_x = [&](u32x4_t (&r)[8], int ci) {
-    const int cc = ci < nchunks ? ci : nchunks - 1;
+  const int xdst0 = ((xr0 >> 5) * 8 + 2 * (xw >> 2)) * kFragB + (xr0 & 31) * 16 + (xw & 3) * 4;
+  const int wb0 = tid >> 5, wt = tid & 31;  // 8-column block within the pass, piece within the block
+  uint32_t wsrc[kWPieces];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(cc) * (kChunkK * 2), 0);
-  };
-  auto store_x = [&](const u32x4_t (&r)[8], int parity) {
-    uint8_t *buf = lds + (parity & 1) * kStageB + xdst0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      // row = r0 + 16 i: row tile i / 2, row within the tile r0 + 16 (i % 2)
-      uint8_t *d = buf + (i >> 1) * (8 * kFragB) + (i & 1) * (16 * 16);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) *reinterpret_cast<uint32_t *>(d + (e >> 1) * kFragB + (e & 1) * (32 * 16)) = r[i][e];
-    }
-  };
+  for (int i = 0; i < kWPieces; ++i) {
+    int nt8 = cb * (kCols / 8) + wb0 + kWTilesPerPass * i;
+    nt8 = nt8 < (N >> 3) ? nt8 : (N >> 3) - 1;
+    wsrc[i] = static_cast<uint32_t>((static_cast<size_t>(nt8) * KT * 32 + wt) * 16);
+  }
+  const int wdst0 = ((wb0 >> 2) * 2 + ((wt & 3) >> 1)) * kFragB + ((wt & 1) * 32 + 8 * (wb0 & 3) + (wt >> 2)) * 16;
 
-  struct WRegs {
-    u32x4_t w[kCT][2];
-    uint32_t s[kCT][NGRP];
+  struct Staged {
+    u32x4_t x[kXPieces], w[kWPieces];
   };
-  auto load_w = [&](WRegs &r, int ci) {
+  auto load_next = [&](Staged &r, int ci) {
     const int cc = ci < nchunks ? ci : nchunks - 1;
-    const uint32_t so = static_cast<uint32_t>(cc) * 512u;
 #pragma unroll
-    for (int ct = 0; ct < kCT; ++ct) {
+    for (int i = 0; i < kXPieces; ++i) r.x[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(cc) * (kChunkK * 2), 0);
 #pragma unroll
-      for (int ld = 0; ld < 2; ++ld) r.w[ct][ld] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[ct][ld], so, 0);
+    for (int i = 0; i < kWPieces; ++i) r.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wsrc[i], static_cast<uint32_t>(cc) * 512u, 0);
+  };
+  auto store_next = [&](const Staged &r, int parity) {
+    uint8_t *bx = lds + (parity & 1) * kStageX + xdst0;
+#pragma unroll
+    for (int i = 0; i < kXPieces; ++i) {
+      uint8_t *d = bx + i * (kXRowsPerPass / 32) * (8 * kFragB);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) *reinterpret_cast<uint32_t *>(d + (e >> 1) * kFragB + (e & 1) * (32 * 16)) = r.x[i][e];
+    }
+    uint8_t *bw = lds_w + (parity & 1) * kStageW + wdst0;
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i) *reinterpret_cast<u32x4_t *>(bw + i * (kWTilesPerPass / 4) * (2 * kFragB)) = r.w[i];
+  };
+  auto load_scales = [&](uint32_t (&r)[kCT][NGRP], int ci) {
+    const int cc = ci < nchunks ? ci : nchunks - 1;
+#pragma unroll
+    for (int ct = 0; ct < kCT; ++ct)
 #pragma unroll
       for (int g = 0; g < NGRP; ++g)
-        r.s[ct][g] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, szlane[ct], static_cast<uint32_t>(cc * NGRP + g) * N * 4u, 0);
-    }
+        r[ct][g] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, szlane[ct], static_cast<uint32_t>(cc * NGRP + g) * N * 4u, 0);
   };
 
   const UnpackConsts uc = unpack_consts();
-  auto compute = [&](const WRegs &r, int parity) {
-    const uint8_t *buf = lds + (parity & 1) * kStageB + (wr * kRT) * (8 * kFragB) + lane * 16;
+  auto compute = [&](const uint32_t (&sc)[kCT][NGRP], int parity) {
+    const uint8_t *bx = lds + (parity & 1) * kStageX + (wr * kRT) * (8 * kFragB) + lane * 16;
+    const uint8_t *bw = lds_w + (parity & 1) * kStageW + (wc * kCT) * (2 * kFragB) + lane * 16;
+    u32x4_t wq[kCT][2];  // [column tile][j pair]: words of the four 32-wide k spans
+#pragma unroll
+    for (int ct = 0; ct < kCT; ++ct)
+#pragma unroll
+      for (int ld = 0; ld < 2; ++ld) wq[ct][ld] = *reinterpret_cast<const u32x4_t *>(bw + (ct * 2 + ld) * kFragB);
 #pragma unroll
     for (int g = 0; g < NGRP; ++g) {
       f32x16_t part[kCT][kRT];
@@ -174,17 +193,17 @@ __global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__rest
         const int s = g * SPG + sg;  // step = 2 p + jp
         bf16x8_t af[kRT];
 #pragma unroll
-        for (int rt = 0; rt < kRT; ++rt) af[rt] = *reinterpret_cast<const bf16x8_t *>(buf + (rt * 8 + s) * kFragB);
+        for (int rt = 0; rt < kRT; ++rt) af[rt] = *reinterpret_cast<const bf16x8_t *>(bx + (rt * 8 + s) * kFragB);
 #pragma unroll
         for (int ct = 0; ct < kCT; ++ct) {
-          const bf16x8_t wf = unpack_word(r.w[ct][s & 1][s >> 1], uc);
+          const bf16x8_t wf = unpack_word(wq[ct][s & 1][s >> 1], uc);
 #pragma unroll
           for (int rt = 0; rt < kRT; ++rt) part[ct][rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[rt], wf, part[ct][rt], 0, 0, 0);
         }
       }
 #pragma unroll
       for (int ct = 0; ct < kCT; ++ct) {
-        const float scale = __builtin_bit_cast(float, r.s[ct][g] << 16);
+        const float scale = __builtin_bit_cast(float, sc[ct][g] << 16);
 #pragma unroll
         for (int rt = 0; rt < kRT; ++rt)
 #pragma unroll
@@ -193,24 +212,24 @@ __global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__rest
     }
   };
 
-  // ---- main loop, two chunks per trip so that the register buffers are compile-time names ------------
-  WRegs ring[2];
-  u32x4_t xst[8];
-  load_x(xst, 0);
-  load_w(ring[0], 0);
-  store_x(xst, 0);
+  // ---- main loop, two chunks per trip so that the scale registers are compile-time names -----------------
+  Staged st;
+  uint32_t sc[2][kCT][NGRP];
+  load_next(st, 0);
+  load_scales(sc[0], 0);
+  store_next(st, 0);
   lds_barrier();
   for (int ci = 0; ci < nchunks; ci += 2) {
-    load_x(xst, ci + 1);
-    load_w(ring[1], ci + 1);
-    compute(ring[0], 0);
-    store_x(xst, 1);
+    load_next(st, ci + 1);       // in flight during the arithmetic of this chunk
+    load_scales(sc[1], ci + 1);
+    compute(sc[0], 0);
+    store_next(st, 1);           // the other stage: everybody left it at the previous barrier
     lds_barrier();
     if (ci + 1 >= nchunks) break;  // uniform
-    load_x(xst, ci + 2);
-    load_w(ring[0], ci + 2);
-    compute(ring[1], 1);
-    store_x(xst, 0);
+    load_next(st, ci + 2);
+    load_scales(sc[0], ci + 2);
+    compute(sc[1], 1);
+    store_next(st, 0);
     lds_barrier();
   }
 
@@ -233,19 +252,20 @@ __global__ __launch_bounds__(256) void int4_gemm32_kernel(const uint16_t *__rest
 int int4_gemm32(const uint16_t *x, const int32_t *packed, const uint16_t *sz, uint16_t *y, const float *xsum, int xsum_stride,
                 int M, int N, int K, int groupsize, hipStream_t stream) {
   if (K % kChunkK != 0 || N % 8 != 0) return E2H_ERR_BAD_SHAPE;
-  const int n_col_blocks = (N + 127) / 128, n_row_blocks = (M + 127) / 128;
+  constexpr int WR = 2, WC = 4;  // 128 rows x 256 columns per workgroup of 8 waves, one workgroup per CU (101 KB of LDS)
+  const int n_col_blocks = (N + 64 * WC - 1) / (64 * WC), n_row_blocks = (M + 64 * WR - 1) / (64 * WR);
   const int cbx = (n_col_blocks + 7) / 8;
   const long long wgs = 8LL * cbx * n_row_blocks;
   if (wgs > 0x7FFFFFFFLL) return E2H_ERR_BAD_SHAPE;
-  // the pre-pass pads its rows to 64; this kernel's lanes read 128-row blocks: rows past the pad return 0 from the
+  // the pre-pass pads its rows to 64; this kernel's lanes read whole row blocks: rows past the pad return 0 from the
   // buffer bound or belong to other groups' rows of the same array -- they only ever reach rows >= M, which are not stored
-  dim3 grid(static_cast<unsigned>(wgs));
+  dim3 grid(static_cast<unsigned>(wgs)), block(64 * WR * WC);
   const uint32_t *w = reinterpret_cast<const uint32_t *>(packed);
   const uint32_t *s = reinterpret_cast<const uint32_t *>(sz);
   switch (groupsize) {
-    case 32: hipLaunchKernelGGL(int4_gemm32_kernel<32>, grid, dim3(256), 0, stream, x, w, s, y, xsum, xsum_stride, M, N, K, n_col_blocks, cbx); break;
-    case 64: hipLaunchKernelGGL(int4_gemm32_kernel<64>, grid, dim3(256), 0, stream, x, w, s, y, xsum, xsum_stride, M, N, K, n_col_blocks, cbx); break;
-    case 128: hipLaunchKernelGGL(int4_gemm32_kernel<128>, grid, dim3(256), 0, stream, x, w, s, y, xsum, xsum_stride, M, N, K, n_col_blocks, cbx); break;
+    case 32: hipLaunchKernelGGL((int4_gemm32_kernel<32, WR, WC>), grid, block, 0, stream, x, w, s, y, xsum, xsum_stride, M, N, K, n_col_blocks, cbx); break;
+    case 64: hipLaunchKernelGGL((int4_gemm32_kernel<64, WR, WC>), grid, block, 0, stream, x, w, s, y, xsum, xsum_stride, M, N, K, n_col_blocks, cbx); break;
+    case 128: hipLaunchKernelGGL((int4_gemm32_kernel<128, WR, WC>), grid, block, 0, stream, x, w, s, y, xsum, xsum_stride, M, N, K, n_col_blocks, cbx); break;
     default: return E2H_ERR_BAD_GROUPSIZE;
   }
   return launch_status();
