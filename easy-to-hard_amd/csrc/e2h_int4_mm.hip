@@ -669,14 +669,15 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   const bool have_ws = workspace && workspace_bytes >= static_cast<int64_t>(kTicketBytes) + (int64_t{1} << 20);
   // Measured on MI355X: 8 waves per workgroup (4 column waves x 2 k-groups, one tile each) is the best
   // all-round shape -- two waves per SIMD overlap arithmetic with memory waits -- and narrow matrices
-  // additionally split K over S workgroups until about 3/4 of the CUs have one.
+  // additionally split K over S workgroups as long as that does not exceed one workgroup per CU (measured: 172
+  // column blocks run faster unsplit than as 344 half-length workgroups; 64 blocks run fastest split four ways).
   Shape sh = {1, 4, 1};
   int s = 1;
   if (wide_ok && mt <= 2) {
     sh = Shape{1, 4, 2};
     const int blocks = ((tiles16 + 3) / 4) * m_chunks;
     if (have_ws)
-      while (s < 4 && blocks * s < (3 * kCUs) / 4 && nchunks / (2 * s * sh.wk) >= 4) s *= 2;
+      while (s < 4 && blocks * s * 2 <= kCUs && nchunks / (2 * s * sh.wk) >= 4) s *= 2;
   } else if (wide_ok) {
     // many rows of x (prefill, scoring): every weight fragment feeds four row tiles straight from registers;
     // wide column blocks keep the LDS traffic for activation fragments below the MFMA rate
