@@ -330,7 +330,7 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
   } else {
     const int blocks = ((tiles16 + 3) / 4) * m_chunks;
     if (have_ws)
-      while (s < 4 && blocks * s < (3 * kCUs8) / 4 && nchunks / (2 * s * wk) >= 4) s *= 2;
+      while (s < 4 && blocks * s * 2 <= kCUs8 && nchunks / (2 * s * wk) >= 4) s *= 2;
   }
   if (options().int8_rows_per_wave == 16 || options().int8_rows_per_wave == 32) t = options().int8_rows_per_wave / 16;
   if (options().int8_k_groups == 1 || options().int8_k_groups == 2) wk = options().int8_k_groups;
