@@ -228,37 +228,47 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict
 // nothing to the caches.  rows_by_token: k / v row = token index t instead of its position (a pass without KV
 // cache, where k and v are fresh tensors of exactly T rows).
 // ------------------------------------------------------------------------------------------------
+// PAIRS = interleaved pairs per thread: 4 (one 16-byte access per tensor, head_dim % 8 == 0) or 1.
+template <int PAIRS>
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ freqs,
                                                             uint16_t *__restrict__ q_out, uint16_t *__restrict__ kc, uint16_t *__restrict__ vc,
-                                                            const int64_t *__restrict__ input_pos, int B, int T, int H, int Hkv, int S, int D, int rows_by_token) {
-  const int pairs_per_row = (H + 2 * Hkv) * D / 2;
+                                                            const int64_t *__restrict__ input_pos, int B, int T, int H, int Hkv, int S, int D,
+                                                            int rows_by_token) {
+  typedef uint32_t vec_t __attribute__((ext_vector_type(PAIRS)));
+  const int units_per_row = (H + 2 * Hkv) * D / (2 * PAIRS);
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= static_cast<int64_t>(B) * T * pairs_per_row) return;
-  const int row = static_cast<int>(idx / pairs_per_row), p = static_cast<int>(idx % pairs_per_row);
+  if (idx >= static_cast<int64_t>(B) * T * units_per_row) return;
+  const int row = static_cast<int>(idx / units_per_row), p = static_cast<int>(idx % units_per_row) * PAIRS;  // first pair
   const int b = row / T, t = row % T;
   const int head = (2 * p) / D, dpair = p % (D / 2);
   const int pos = static_cast<int>(input_pos[t]);   // rotation angle
   const int slot = rows_by_token ? t : pos;         // row of the k / v tensors that receives this token
   const bool pos_ok = pos >= 0 && slot >= 0 && slot < S;
-  const uint32_t raw = reinterpret_cast<const uint32_t *>(qkv)[idx];
-  const float x0 = __builtin_bit_cast(float, raw << 16), x1 = __builtin_bit_cast(float, raw & 0xFFFF0000u);
+  const vec_t raw = reinterpret_cast<const vec_t *>(qkv)[idx];
   if (head < H + Hkv) {
     if (!pos_ok) return;  // no angle for such a position
-    const uint32_t f = reinterpret_cast<const uint32_t *>(freqs)[static_cast<size_t>(pos) * (D / 2) + dpair];
-    const float cs = __builtin_bit_cast(float, f << 16), sn = __builtin_bit_cast(float, f & 0xFFFF0000u);
-    // two separately rounded products and their difference / sum, as torch evaluates the expression in float32
-    const float r0 = x0 * cs - x1 * sn;
-    const float r1 = x1 * cs + x0 * sn;
-    const uint32_t o = static_cast<uint32_t>(f32_to_bf16_rne(r0)) | (static_cast<uint32_t>(f32_to_bf16_rne(r1)) << 16);
+    const vec_t f = *reinterpret_cast<const vec_t *>(reinterpret_cast<const uint32_t *>(freqs) + static_cast<size_t>(pos) * (D / 2) + dpair);
+    vec_t o;
+#pragma unroll
+    for (int i = 0; i < PAIRS; ++i) {
+      const uint32_t ri = raw[i], fi = f[i];
+      const float x0 = __builtin_bit_cast(float, ri << 16), x1 = __builtin_bit_cast(float, ri & 0xFFFF0000u);
+      const float cs = __builtin_bit_cast(float, fi << 16), sn = __builtin_bit_cast(float, fi & 0xFFFF0000u);
+      // two separately rounded products and their difference / sum, as torch evaluates the expression in float32
+      const float r0 = x0 * cs - x1 * sn;
+      const float r1 = x1 * cs + x0 * sn;
+      const uint32_t oi = static_cast<uint32_t>(f32_to_bf16_rne(r0)) | (static_cast<uint32_t>(f32_to_bf16_rne(r1)) << 16);
+      o[i] = oi;
+    }
     if (head < H) {
-      reinterpret_cast<uint32_t *>(q_out)[((static_cast<size_t>(b) * H + head) * T + t) * (D / 2) + dpair] = o;
+      *reinterpret_cast<vec_t *>(reinterpret_cast<uint32_t *>(q_out) + ((static_cast<size_t>(b) * H + head) * T + t) * (D / 2) + dpair) = o;
     } else {
       const int hk = head - H;
-      reinterpret_cast<uint32_t *>(kc)[((static_cast<size_t>(b) * Hkv + hk) * S + slot) * (D / 2) + dpair] = o;
+      *reinterpret_cast<vec_t *>(reinterpret_cast<uint32_t *>(kc) + ((static_cast<size_t>(b) * Hkv + hk) * S + slot) * (D / 2) + dpair) = o;
     }
   } else if (pos_ok) {
     const int hk = head - H - Hkv;
-    reinterpret_cast<uint32_t *>(vc)[((static_cast<size_t>(b) * Hkv + hk) * S + slot) * (D / 2) + dpair] = raw;
+    *reinterpret_cast<vec_t *>(reinterpret_cast<uint32_t *>(vc) + ((static_cast<size_t>(b) * Hkv + hk) * S + slot) * (D / 2) + dpair) = raw;
   }
 }
 
@@ -345,8 +355,15 @@ extern "C" int e2h_rope_kv_write_seq(const uint16_t *qkv, const uint16_t *freqs_
   if ((reinterpret_cast<uintptr_t>(qkv) & 3u) || (reinterpret_cast<uintptr_t>(freqs_cis) & 3u) || (reinterpret_cast<uintptr_t>(q_out) & 3u) ||
       (reinterpret_cast<uintptr_t>(k_cache) & 3u) || (reinterpret_cast<uintptr_t>(v_cache) & 3u) || (reinterpret_cast<uintptr_t>(input_pos) & 7u))
     return E2H_ERR_MISALIGNED;
-  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), qkv,
-                     freqs_cis, q_out, k_cache, v_cache, input_pos, (int)batch, (int)seqlen, (int)n_head, (int)n_kv_head, (int)cache_len, (int)head_dim, rows_by_token ? 1 : 0);
+  const bool vec = (head_dim % 8) == 0 && !((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(freqs_cis) | reinterpret_cast<uintptr_t>(q_out) |
+                                            reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15u);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (vec)
+    hipLaunchKernelGGL(rope_kv_write_kernel<4>, dim3(static_cast<unsigned>((pairs / 4 + 255) / 256)), dim3(256), 0, st, qkv, freqs_cis, q_out, k_cache,
+                       v_cache, input_pos, (int)batch, (int)seqlen, (int)n_head, (int)n_kv_head, (int)cache_len, (int)head_dim, rows_by_token ? 1 : 0);
+  else
+    hipLaunchKernelGGL(rope_kv_write_kernel<1>, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, st, qkv, freqs_cis, q_out, k_cache,
+                       v_cache, input_pos, (int)batch, (int)seqlen, (int)n_head, (int)n_kv_head, (int)cache_len, (int)head_dim, rows_by_token ? 1 : 0);
   return launch_status();
 }
 
