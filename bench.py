@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--per-shape", default="",
                     help="comma-separated row counts M: time every distinct quantized-linear shape of the model at each M "
                          "(all layers' instances back to back, so the weights rotate) and print one JSON line")
+    ap.add_argument("--stock", action="store_true",
+                    help="with --per-shape (int4): time PyTorch-ROCm's own aten._weight_int4pack_mm on the same codes instead "
+                         "of this library's kernel, and report the largest difference between the two results")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch-geometry override passed to e2h_set_option (experiments)")
     ap.add_argument("--gemv-only", action="store_true",
@@ -151,7 +154,19 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
     }
 
 
-def measure_per_shape(model, rows_list, reps=6):
+def stock_int4_operands(mod):
+    """The same codes and (scale, zero) pairs in the form PyTorch-ROCm's own aten._weight_int4pack_mm takes (its packing
+    differs from the checkpoint layout): codes two per byte, even k in the high nibble, through its own packer."""
+    import torch
+
+    from easy_to_hard_amd import ops
+
+    codes = ops.int4_unpack(mod.weight)
+    two_per_byte = ((codes[:, ::2] << 4) | codes[:, 1::2]).to(torch.uint8)
+    return torch.ops.aten._convert_weight_to_int4pack(two_per_byte, mod.inner_k_tiles), mod.scales_and_zeros
+
+
+def measure_per_shape(model, rows_list, reps=6, stock=False):
     """Average launch duration of each distinct quantized-linear shape, replayed from a HIP graph and timed with events on
     the launch stream; the instances of a shape in different layers have different weights, so nothing stays cached."""
     import torch
@@ -167,10 +182,20 @@ def measure_per_shape(model, rows_list, reps=6):
         for m in rows_list:
             x = torch.randn((m, k), device=dev, dtype=torch.float32).to(torch.bfloat16)
 
+            stock_ops = [stock_int4_operands(mod) for mod in mods] if stock else None
+
             def one_pass():
+                if stock_ops is not None:
+                    for (w_stock, sz), mod in zip(stock_ops, mods):
+                        torch.ops.aten._weight_int4pack_mm(x, w_stock, mod.groupsize, sz)
+                    return
                 for mod in mods:
                     mod(x)
 
+            if stock_ops is not None:  # same codes, so the two kernels must agree to bf16 rounding
+                y_stock = torch.ops.aten._weight_int4pack_mm(x, stock_ops[0][0], mods[0].groupsize, stock_ops[0][1]).float()
+                y_ours = mods[0](x).float()
+                stock_err = float((y_stock - y_ours).abs().max() / y_ours.abs().max())
             side = torch.cuda.Stream(device=dev)
             side.wait_stream(torch.cuda.current_stream(dev))
             with torch.cuda.stream(side):
@@ -194,6 +219,9 @@ def measure_per_shape(model, rows_list, reps=6):
             out.append({"linear": leaf, "n": n, "k": k, "m": m, "instances": len(mods), "us": round(us, 2),
                         "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
                         "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "kind": "int4" if int4 else "int8"})
+            if stock_ops is not None:
+                out[-1]["kernel"] = "aten._weight_int4pack_mm"
+                out[-1]["max_diff_vs_e2h"] = round(stock_err, 5)
     return out
 
 
@@ -319,7 +347,7 @@ def main():
     batch, t_prompt = args.batch, args.prompt
     if args.per_shape:
         rows_list = [int(v) for v in args.per_shape.split(",") if v]
-        print(json.dumps({"per_shape": measure_per_shape(model, rows_list), "model": args.model, "mode": args.mode,
+        print(json.dumps({"per_shape": measure_per_shape(model, rows_list, stock=args.stock), "model": args.model, "mode": args.mode,
                           "groupsize": args.groupsize if args.mode == "int4" else None}))
         return
     if args.gemv_only:

@@ -427,3 +427,27 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k):
     assert torch.equal(yi, yi2)
     y_rr = qo.int8_linear_reference_rounding(bf16_to_np(xi), q, s)
     assert np.array_equal(bf16_to_np(yi), y_rr)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m", [1, 32])
+def test_int4_mm_matches_the_stock_rocm_op_on_identical_codes(m):
+    """PyTorch-ROCm ships its own aten._weight_int4pack_mm (another packed layout, same arithmetic: the op the reference
+    calls at models/quantize.py:448-450).  Fed the same codes and (scale, zero) pairs it must agree with this library to
+    bfloat16 rounding; skipped where the installed build has no kernel for this GPU."""
+    dev = "cuda:0"
+    gen = torch.Generator().manual_seed(99)
+    n, k, g, ikt = 512, 1024, 128, 8
+    w = (torch.randn((n, k), generator=gen) * 0.02).to(torch.bfloat16).to(dev)
+    x = torch.randn((m, k), generator=gen).to(torch.bfloat16).to(dev)
+    packed, sz = e2h.prepare_int4_weight_and_scales_and_zeros(w, g, ikt)
+    codes = ops.int4_unpack(packed)
+    two_per_byte = ((codes[:, ::2] << 4) | codes[:, 1::2]).to(torch.uint8)
+    try:
+        stock_packed = torch.ops.aten._convert_weight_to_int4pack(two_per_byte, ikt)
+        y_stock = torch.ops.aten._weight_int4pack_mm(x, stock_packed, g, sz).float()
+        torch.cuda.synchronize()
+    except (RuntimeError, NotImplementedError) as exc:
+        pytest.skip(f"stock aten._weight_int4pack_mm unavailable here: {exc}")
+    y = ops.int4_mm_direct(x, packed, g, sz).float()
+    assert float((y - y_stock).abs().max() / y_stock.abs().max()) <= 1e-2
