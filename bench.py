@@ -55,6 +55,10 @@ def parse_args():
     ap.add_argument("--stock", action="store_true",
                     help="with --per-shape (int4): time PyTorch-ROCm's own aten._weight_int4pack_mm on the same codes instead "
                          "of this library's kernel, and report the largest difference between the two results")
+    ap.add_argument("--stock-step", action="store_true",
+                    help="comparator run of the decode benchmark: the same model and HIP-graph replayed step, but every int4 "
+                         "linear goes through PyTorch-ROCm's aten._weight_int4pack_mm and everything around the linears through "
+                         "stock torch ops (what the reference's model code executes, without inductor); prints its own JSON line")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch-geometry override passed to e2h_set_option (experiments)")
     ap.add_argument("--gemv-only", action="store_true",
@@ -361,6 +365,17 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"roofline": roofline, "calibration_copy_bytes": src.numel()}))
         return
+    if args.stock_step:
+        import easy_to_hard_amd as e2h
+        import easy_to_hard_amd.model as model_mod
+
+        assert args.mode == "int4", "--stock-step compares the int4 path"
+        model_mod.FUSED_DECODE = False
+        for _, mod in quantized_linears(model):
+            if isinstance(mod, e2h.WeightOnlyInt4Linear):
+                w_stock, sz = stock_int4_operands(mod)
+                mod.forward = (lambda x, w=w_stock, q=sz, g=mod.groupsize, n=mod.out_features:
+                               torch.ops.aten._weight_int4pack_mm(x.reshape(-1, x.shape[-1]), w, g, q).reshape(*x.shape[:-1], n))
     max_seq = min(t_prompt + args.max_new, cfg.block_size)
     assert args.warmup + args.steps < max_seq - t_prompt, "warmup + steps must fit in the decode budget"
     model.setup_caches(batch, max_seq)
@@ -385,6 +400,12 @@ def main():
     elapsed = time.perf_counter() - t0
     tok_s = batch * args.steps / elapsed
 
+    if args.stock_step:
+        print(json.dumps({"comparator": "stock torch ops + aten._weight_int4pack_mm, HIP-graph replayed decode step",
+                          "value": round(tok_s, 2), "unit": "tok/s", "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+                          "steps": args.steps, "warmup": args.warmup, "batch": batch, "prompt_len": t_prompt, "model": args.model,
+                          "groupsize": args.groupsize}))
+        return
     roofline = measure_gemv_roofline(model, batch, args.gemv_reps, (args.model, args.mode, args.groupsize, batch))
     cpu = None if args.no_cpu_baseline else measure_cpu_baseline(model, batch, args.groupsize)
 
