@@ -82,5 +82,10 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.row_tiles = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "attention_waves")) {
+    if (value != 0 && value != 4 && value != 8) return E2H_ERR_BAD_OPTION;
+    o.attention_waves = value;
+    return E2H_OK;
+  }
   return E2H_ERR_BAD_OPTION;
 }

@@ -19,14 +19,14 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // ------------------------------------------------------------------------------------------------
 // decode attention: q [B, H, D], caches [Bmax, Hkv, S, D] bf16, out [B, H, D] bf16.
-// One workgroup (4 waves) per (b, kv head); the waves split the live positions, every wave keeps REP query heads
+// One workgroup (NW = 4 or 8 waves) per (b, kv head); the waves split the live positions, every wave keeps REP query heads
 // (the heads that share the kv head) so that each K / V row is loaded once.  Lane layout: LPP = D/8 lanes cover
 // one position (16 bytes each), a wave-wide load covers 64/LPP positions.  Online softmax in float32.
 // Visible positions: t <= pos, and if left_pad is given additionally (t >= left_pad[b] or t == pos)
 // (reference models/model.py:221-228).
 // ------------------------------------------------------------------------------------------------
-template <int D, int REP>
-__global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
+template <int D, int REP, int NW>
+__global__ __launch_bounds__(64 * NW) void decode_attention_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
                                                                const uint16_t *__restrict__ vc, uint16_t *__restrict__ out,
                                                                const int64_t *__restrict__ input_pos, const int64_t *__restrict__ left_pad,
                                                                int H, int Hkv, int S, float scale) {
@@ -64,17 +64,25 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *_
     for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
   }
 
-  // waves take interleaved tiles of UNR * PPL positions
-  for (int t0 = wave * (UNR * PPL); t0 < n_live; t0 += 4 * UNR * PPL) {
-    u32x4_t kr[UNR], vr[UNR];
-    int tpos[UNR];
+  // waves take interleaved tiles of UNR * PPL positions; the rows of a wave's next tile are requested before the
+  // current tile is worked on, so a wave has two tiles in flight instead of one HBM round trip per tile
+  auto fetch = [&](int t0, u32x4_t (&kr)[UNR], u32x4_t (&vr)[UNR]) {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      tpos[u] = t0 + u * PPL + pg;
-      const int tc = tpos[u] < n_live ? tpos[u] : n_live - 1;
+      const int tp = t0 + u * PPL + pg;
+      const int tc = tp < n_live ? tp : n_live - 1;
       kr[u] = *reinterpret_cast<const u32x4_t *>(kbase + static_cast<size_t>(tc) * D);
       vr[u] = *reinterpret_cast<const u32x4_t *>(vbase + static_cast<size_t>(tc) * D);
     }
+  };
+  u32x4_t kr[UNR], vr[UNR], kn[UNR], vn[UNR];
+  if (wave * (UNR * PPL) < n_live) fetch(wave * (UNR * PPL), kr, vr);
+  for (int t0 = wave * (UNR * PPL); t0 < n_live; t0 += NW * UNR * PPL) {
+    const bool more = t0 + NW * UNR * PPL < n_live;
+    if (more) fetch(t0 + NW * UNR * PPL, kn, vn);
+    int tpos[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) tpos[u] = t0 + u * PPL + pg;
     float s[REP][UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
@@ -119,10 +127,17 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *_
         }
       }
     }
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        kr[u] = kn[u];
+        vr[u] = vn[u];
+      }
+    }
   }
 
   // combine the position groups of a wave, then the waves
-  __shared__ float sh_m[4][REP], sh_l[4][REP], sh_acc[4][REP][D];
+  __shared__ float sh_m[NW][REP], sh_l[NW][REP], sh_acc[NW][REP][D];
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
     // l_run counts each position once per lane of its group (every lane of the group holds the same p): sum over groups
@@ -146,14 +161,14 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(const uint16_t *_
     }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < REP * D; e += 256) {
+  for (int e = threadIdx.x; e < REP * D; e += 64 * NW) {
     const int r = e / D, d = e % D;
     float m = sh_m[0][r];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) m = fmaxf(m, sh_m[w][r]);
+    for (int w = 1; w < NW; ++w) m = fmaxf(m, sh_m[w][r]);
     float l = 0.f, a = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float c = __expf(sh_m[w][r] - m);
       l += sh_l[w][r] * c;
       a += sh_acc[w][r][d] * c;
@@ -290,17 +305,27 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
   reinterpret_cast<u32x4_t *>(y)[idx] = o;
 }
 
-template <int D>
-int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
-                     const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
+template <int D, int NW>
+int launch_attention_nw(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
+                        const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
   switch (rep) {
-    case 1: hipLaunchKernelGGL((decode_attention_kernel<D, 1>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
-    case 2: hipLaunchKernelGGL((decode_attention_kernel<D, 2>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
-    case 4: hipLaunchKernelGGL((decode_attention_kernel<D, 4>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
-    case 8: hipLaunchKernelGGL((decode_attention_kernel<D, 8>), grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 1: hipLaunchKernelGGL((decode_attention_kernel<D, 1, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 2: hipLaunchKernelGGL((decode_attention_kernel<D, 2, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 4: hipLaunchKernelGGL((decode_attention_kernel<D, 4, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 8: hipLaunchKernelGGL((decode_attention_kernel<D, 8, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
     default: return E2H_ERR_BAD_SHAPE;
   }
   return launch_status();
+}
+
+// The live length is a device value (graph replays move it), so the waves per workgroup follow the cache length:
+// eight waves for caches beyond 256 positions halve the tiles a wave walks through one after the other.
+template <int D>
+int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
+                     const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
+  const int nw = options().attention_waves ? options().attention_waves : (S > 256 ? 8 : 4);
+  if (nw == 8) return launch_attention_nw<D, 8>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale);
+  return launch_attention_nw<D, 4>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale);
 }
 
 }  // namespace

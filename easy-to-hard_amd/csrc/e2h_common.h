@@ -47,6 +47,7 @@ struct Options {
   int int4_no_gemm32;      // 1 = many-row calls (int4 and int8) stay on the 16x16-tile kernels
   int int4_gemm32_min_rows;  // 0 = by workgroup count, else rows from which the 32x32-tile kernels take over
   int row_tiles;           // 0 = heuristic, else 1/2/4 tiles of 16 activation rows per workgroup (both matmuls)
+  int attention_waves;     // 0 = by cache length, else 4 or 8 waves per decode-attention workgroup
 };
 Options &options();
 
