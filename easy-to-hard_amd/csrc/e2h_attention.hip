@@ -180,59 +180,94 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_kernel(const uint16_
 // ------------------------------------------------------------------------------------------------
 // RMSNorm (reference :363-377): bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w), float32 statistics.
 // ------------------------------------------------------------------------------------------------
-// One workgroup per row.  With `delta` the kernel first forms h = bf16(x + delta) (the residual add of
-// TransformerBlock.forward, reference :279-282), stores it to h_out and normalises h.
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ delta,
-                                                      const uint16_t *__restrict__ w, uint16_t *__restrict__ h_out,
-                                                      uint16_t *__restrict__ y, int dim, float eps) {
+// One workgroup of BLOCK threads per row.  With `delta` the kernel first forms h = bf16(x + delta) (the residual add
+// of TransformerBlock.forward, reference :279-282), stores it to h_out and normalises h.  The first kPieces pieces of
+// 8 values per thread stay in registers and all their loads are issued before anything is waited for (one memory
+// round trip for the whole row up to BLOCK * 8 * kPieces values); longer rows re-read the rest.
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ delta,
+                                                        const uint16_t *__restrict__ w, uint16_t *__restrict__ h_out,
+                                                        uint16_t *__restrict__ y, int dim, float eps) {
+  constexpr int kPieces = 2, kStride = BLOCK * 8, kWaves = BLOCK / 64;
   const size_t row = blockIdx.x;
   const uint16_t *xr = x + row * dim;
-  constexpr int kMaxPieces = 4;  // dim <= 256 * 8 * 4 = 8192 values are kept in registers, longer rows are re-read
-  u32x4_t keep[kMaxPieces], keepw[kMaxPieces];
-  float ss = 0.f;
-  int np = 0;
-  for (int i = threadIdx.x * 8; i < dim; i += 2048, ++np) {
-    u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
-    if (np < kMaxPieces) keepw[np] = *reinterpret_cast<const u32x4_t *>(w + i);  // in flight across the reduction
-    if (delta) {
-      const u32x4_t dr = *reinterpret_cast<const u32x4_t *>(delta + row * dim + i);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float a = __builtin_bit_cast(float, raw[j] << 16) + __builtin_bit_cast(float, dr[j] << 16);
-        const float bq = __builtin_bit_cast(float, raw[j] & 0xFFFF0000u) + __builtin_bit_cast(float, dr[j] & 0xFFFF0000u);
-        raw[j] = static_cast<uint32_t>(f32_to_bf16_rne(a)) | (static_cast<uint32_t>(f32_to_bf16_rne(bq)) << 16);
-      }
-      *reinterpret_cast<u32x4_t *>(h_out + row * dim + i) = raw;
-    }
-    if (np < kMaxPieces) keep[np] = raw;
+  const uint16_t *dr_row = delta ? delta + row * dim : nullptr;
+  auto add_round = [](u32x4_t a, u32x4_t d) {  // bf16(x + delta), value by value
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float a = __builtin_bit_cast(float, raw[j] << 16), bq = __builtin_bit_cast(float, raw[j] & 0xFFFF0000u);
-      ss = __builtin_fmaf(a, a, ss);
-      ss = __builtin_fmaf(bq, bq, ss);
+      const float lo = __builtin_bit_cast(float, a[j] << 16) + __builtin_bit_cast(float, d[j] << 16);
+      const float hi = __builtin_bit_cast(float, a[j] & 0xFFFF0000u) + __builtin_bit_cast(float, d[j] & 0xFFFF0000u);
+      a[j] = static_cast<uint32_t>(f32_to_bf16_rne(lo)) | (static_cast<uint32_t>(f32_to_bf16_rne(hi)) << 16);
     }
-  }
-  ss = wave_sum(ss);
-  __shared__ float part[4];
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
-  __syncthreads();
-  ss = (part[0] + part[1]) + (part[2] + part[3]);
-  const float inv = rsqrtf(ss / static_cast<float>(dim) + eps);
-  const uint16_t *src = delta ? h_out + row * dim : xr;
-  uint16_t *yr = y + row * dim;
-  np = 0;
-  for (int i = threadIdx.x * 8; i < dim; i += 2048, ++np) {
-    const u32x4_t raw = np < kMaxPieces ? keep[np] : *reinterpret_cast<const u32x4_t *>(src + i);
-    const u32x4_t wr = np < kMaxPieces ? keepw[np] : *reinterpret_cast<const u32x4_t *>(w + i);
+    return a;
+  };
+  auto sum_sq = [](u32x4_t a, float ss) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float lo = __builtin_bit_cast(float, a[j] << 16), hi = __builtin_bit_cast(float, a[j] & 0xFFFF0000u);
+      ss = __builtin_fmaf(lo, lo, ss);
+      ss = __builtin_fmaf(hi, hi, ss);
+    }
+    return ss;
+  };
+  auto scale_store = [&](u32x4_t raw, u32x4_t wr, float inv, uint16_t *dst) {
     u32x4_t o;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float a = bf16_round(__builtin_bit_cast(float, raw[j] << 16) * inv) * __builtin_bit_cast(float, wr[j] << 16);
-      const float bq = bf16_round(__builtin_bit_cast(float, raw[j] & 0xFFFF0000u) * inv) * __builtin_bit_cast(float, wr[j] & 0xFFFF0000u);
-      o[j] = static_cast<uint32_t>(f32_to_bf16_rne(a)) | (static_cast<uint32_t>(f32_to_bf16_rne(bq)) << 16);
+      const float lo = bf16_round(__builtin_bit_cast(float, raw[j] << 16) * inv) * __builtin_bit_cast(float, wr[j] << 16);
+      const float hi = bf16_round(__builtin_bit_cast(float, raw[j] & 0xFFFF0000u) * inv) * __builtin_bit_cast(float, wr[j] & 0xFFFF0000u);
+      o[j] = static_cast<uint32_t>(f32_to_bf16_rne(lo)) | (static_cast<uint32_t>(f32_to_bf16_rne(hi)) << 16);
     }
-    *reinterpret_cast<u32x4_t *>(yr + i) = o;
+    *reinterpret_cast<u32x4_t *>(dst) = o;
+  };
+
+  u32x4_t keep[kPieces], keepd[kPieces], keepw[kPieces];
+#pragma unroll
+  for (int p = 0; p < kPieces; ++p) {
+    const int i = threadIdx.x * 8 + p * kStride;
+    if (i < dim) {
+      keep[p] = *reinterpret_cast<const u32x4_t *>(xr + i);
+      if (delta) keepd[p] = *reinterpret_cast<const u32x4_t *>(dr_row + i);
+      keepw[p] = *reinterpret_cast<const u32x4_t *>(w + i);  // needed only after the reduction
+    }
   }
+  float ss = 0.f;
+#pragma unroll
+  for (int p = 0; p < kPieces; ++p) {
+    const int i = threadIdx.x * 8 + p * kStride;
+    if (i < dim) {
+      if (delta) {
+        keep[p] = add_round(keep[p], keepd[p]);
+        *reinterpret_cast<u32x4_t *>(h_out + row * dim + i) = keep[p];
+      }
+      ss = sum_sq(keep[p], ss);
+    }
+  }
+  for (int i = threadIdx.x * 8 + kPieces * kStride; i < dim; i += kStride) {
+    u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
+    if (delta) {
+      raw = add_round(raw, *reinterpret_cast<const u32x4_t *>(dr_row + i));
+      *reinterpret_cast<u32x4_t *>(h_out + row * dim + i) = raw;
+    }
+    ss = sum_sq(raw, ss);
+  }
+  ss = wave_sum(ss);
+  __shared__ float part[kWaves];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();  // also makes this thread's own h_out stores visible to its re-reads below
+  ss = 0.f;
+#pragma unroll
+  for (int wv = 0; wv < kWaves; ++wv) ss += part[wv];
+  const float inv = rsqrtf(ss / static_cast<float>(dim) + eps);
+  const uint16_t *src = delta ? h_out + row * dim : xr;
+  uint16_t *yr = y + row * dim;
+#pragma unroll
+  for (int p = 0; p < kPieces; ++p) {
+    const int i = threadIdx.x * 8 + p * kStride;
+    if (i < dim) scale_store(keep[p], keepw[p], inv, yr + i);
+  }
+  for (int i = threadIdx.x * 8 + kPieces * kStride; i < dim; i += kStride)
+    scale_store(*reinterpret_cast<const u32x4_t *>(src + i), *reinterpret_cast<const u32x4_t *>(w + i), inv, yr + i);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -305,6 +340,15 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
   reinterpret_cast<u32x4_t *>(y)[idx] = o;
 }
 
+// few rows (decode): 512 threads so that a 4096-wide row is one piece per thread; many rows: 256-thread workgroups
+void launch_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *w, uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim,
+                    float eps, hipStream_t stream) {
+  if (rows <= 512 && dim >= 4096)
+    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(static_cast<unsigned>(rows)), dim3(512), 0, stream, x, delta, w, h_out, y, static_cast<int>(dim), eps);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, x, delta, w, h_out, y, static_cast<int>(dim), eps);
+}
+
 template <int D, int NW>
 int launch_attention_nw(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
                         const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
@@ -354,8 +398,7 @@ extern "C" int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *
   if (!x || !weight || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream), x, nullptr, weight, nullptr,
-                     y, static_cast<int>(dim), eps);
+  launch_rmsnorm(x, nullptr, weight, nullptr, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 
@@ -364,8 +407,7 @@ extern "C" int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const u
   if (!x || !delta || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(delta) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream), x, delta, weight, h_out,
-                     y, static_cast<int>(dim), eps);
+  launch_rmsnorm(x, delta, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 

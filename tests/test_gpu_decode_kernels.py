@@ -15,29 +15,36 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def _rmsnorm_reference(x, w, eps):
+    """RMSNorm with the reference's rounding points (models/model.py:363-377) on stock ops.  mean(x^2) depends on the
+    summation order in its last float32 bit, and where x * rsqrt(..) sits next to a bfloat16 rounding boundary that bit
+    flips the first rounding and, through the multiplication by w, up to two ulps of the result (a whole row of 4096
+    can do so when rsqrt(..) happens to be close to a short binary fraction): hence two ulps of tolerance and an
+    "almost everywhere identical" check rather than equality."""
+    xf = x.float()
+    return (xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + eps)).to(torch.bfloat16) * w
+
+
 def test_rmsnorm_matches_stock_ops():
-    for rows, dim in [(32, 4096), (5, 256), (1, 8192), (70, 512), (2, 16384)]:
+    for rows, dim in [(32, 4096), (5, 256), (1, 8192), (70, 512), (2, 16384), (600, 4096), (3, 20480)]:
         x = randn_bf16((rows, dim), std=1.5, seed=rows).to(DEV)
         w = (1 + 0.1 * randn_bf16((dim,), seed=dim).float()).to(torch.bfloat16).to(DEV)
-        xf = x.float()
-        ref = (xf * torch.rsqrt(torch.mean(xf * xf, dim=-1, keepdim=True) + 1e-5)).to(torch.bfloat16) * w
+        ref = _rmsnorm_reference(x, w, 1e-5)
         y = ops.rmsnorm(x, w, 1e-5)
-        # identical up to the summation order of mean(x^2): at most one bf16 ulp, almost always zero
-        assert torch.allclose(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+        assert torch.allclose(y.float(), ref.float(), rtol=2 ** -6, atol=1e-6)
         assert (y == ref).float().mean() > 0.99
 
 
 def test_add_rmsnorm_matches_stock_ops():
-    for rows, dim in [(32, 4096), (3, 256), (2, 16384)]:
+    for rows, dim in [(32, 4096), (3, 256), (2, 16384), (600, 4096), (3, 20480)]:
         x = randn_bf16((rows, dim), std=1.5, seed=rows).to(DEV)
         d = randn_bf16((rows, dim), std=0.7, seed=rows + 1).to(DEV)
         w = (1 + 0.1 * randn_bf16((dim,), seed=dim).float()).to(torch.bfloat16).to(DEV)
         h_ref = x + d
-        hf = h_ref.float()
-        ref = (hf * torch.rsqrt(torch.mean(hf * hf, dim=-1, keepdim=True) + 1e-5)).to(torch.bfloat16) * w
+        ref = _rmsnorm_reference(h_ref, w, 1e-5)
         h, y = ops.add_rmsnorm(x, d, w, 1e-5)
         assert torch.equal(h, h_ref)
-        assert torch.allclose(y.float(), ref.float(), rtol=2 ** -7, atol=1e-6)
+        assert torch.allclose(y.float(), ref.float(), rtol=2 ** -6, atol=1e-6)
         assert (y == ref).float().mean() > 0.99
 
 
