@@ -222,12 +222,14 @@ __global__ __launch_bounds__(64 * WR * WC) void int4_gemm32_kernel(const uint16_
   for (int ci = 0; ci < nchunks; ci += 2) {
     load_next(st, ci + 1);       // in flight during the arithmetic of this chunk
     load_scales(sc[1], ci + 1);
+    __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic: the scheduler would sink it to its first use
     compute(sc[0], 0);
     store_next(st, 1);           // the other stage: everybody left it at the previous barrier
     lds_barrier();
     if (ci + 1 >= nchunks) break;  // uniform
     load_next(st, ci + 2);
     load_scales(sc[0], ci + 2);
+    __builtin_amdgcn_sched_barrier(0);
     compute(sc[1], 1);
     store_next(st, 0);
     lds_barrier();

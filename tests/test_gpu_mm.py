@@ -398,11 +398,13 @@ def test_int4_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, g):
     assert (yi.float() - yi2.float()).abs().max().item() <= 2.0 ** -7 * yi2.float().abs().max().item()
 
 
-@pytest.mark.parametrize("m,n,k", [(65, 1, 128), (130, 272, 1024), (257, 136, 384), (512, 4096, 4096), (300, 2, 4096)])
-def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k):
-    """The 32x32-tile int8 kernel (many rows) against the oracle, the reference's two-rounding form and the
-    16x16-tile kernel: ragged M and N (incl. the 2-row reward head), a single chunk, odd chunk counts, and rows
-    with extreme codes (-128 / 127) so that the +128 offset and its correction are exercised at both ends."""
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("m,n,k", [(65, 1, 128), (130, 272, 1024), (257, 136, 384), (512, 4096, 4096), (300, 2, 4096), (700, 520, 640)])
+def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile):
+    """The 32x32-tile int8 kernels (many rows; 128 x 256 and 256 x 256 outputs per workgroup) against the oracle, the
+    reference's two-rounding form and the 16x16-tile kernel: ragged M and N (incl. the 2-row reward head), a single
+    chunk, odd chunk counts, and rows with extreme codes (-128 / 127) so that the +128 offset and its correction are
+    exercised at both ends."""
     q, s, q_d, s_d = _int8_case(n, k, seed=m + n)
     q = q.copy()
     q[0, :4] = (-128, 127, -128, 127)
@@ -410,12 +412,14 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k):
     q_d = torch.from_numpy(q).to(DEV)
     x = randn_bf16((m, k), std=1.0, seed=m + 2)
     _lib.set_option("int4_gemm32_min_rows", 65)
+    _lib.set_option("int8_gemm_tile", tile)
     try:
         y, _ = _check_int8(x, q, s, q_d, s_d)
         xi = torch.randint(-1, 2, (m, k), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
         yi = ops.int8_mm_direct(xi.to(DEV), q_d, s_d)
     finally:
         _lib.set_option("int4_gemm32_min_rows", 0)
+        _lib.set_option("int8_gemm_tile", 0)
     _lib.set_option("int4_no_gemm32", 1)
     try:
         y2, _ = _check_int8(x, q, s, q_d, s_d)
