@@ -148,8 +148,64 @@ __global__ __launch_bounds__(kSampleThreads) void sample_top_k_kernel(const uint
   }
 }
 
+// Greedy choice: argmax(float(logits)) per row (reference inference_generate.py: the temperature-0 / greedy path of the
+// harness, torch.argmax over the last position's logits).  Ties go to the lowest index and a NaN counts as the
+// largest value, as in ATen's arg-max reduction.  One workgroup per row, 16-byte loads where the row allows them.
+__device__ __forceinline__ uint32_t argmax_key(uint32_t bf16_bits) {  // larger value <=> larger key, NaN above +inf
+  const uint32_t u = bf16_bits << 16;
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0xFFFFFFFFu;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__global__ __launch_bounds__(kSampleThreads) void argmax_rows_kernel(const uint16_t *__restrict__ logits, int64_t row_stride,
+                                                                     int64_t *__restrict__ out, int vocab) {
+  __shared__ unsigned long long s_best[kSampleThreads / 64];
+  const uint16_t *row = logits + static_cast<size_t>(blockIdx.x) * row_stride;
+  // candidate = (key << 32) | ~index: the maximum is the largest key and, among equals, the smallest index
+  unsigned long long best = 0ull;
+  auto offer = [&](uint32_t bits, int i) {
+    const unsigned long long cand = (static_cast<unsigned long long>(argmax_key(bits)) << 32) | static_cast<uint32_t>(~static_cast<uint32_t>(i));
+    best = cand > best ? cand : best;
+  };
+  if ((reinterpret_cast<uintptr_t>(row) & 15u) == 0) {
+    const int pieces = vocab / 8;
+    for (int p = threadIdx.x; p < pieces; p += kSampleThreads) {
+      const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(row + p * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        offer(raw[j] & 0xFFFFu, p * 8 + 2 * j);
+        offer(raw[j] >> 16, p * 8 + 2 * j + 1);
+      }
+    }
+    for (int i = pieces * 8 + threadIdx.x; i < vocab; i += kSampleThreads) offer(row[i], i);
+  } else {
+    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) offer(row[i], i);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned long long other = __shfl_xor(best, off);
+    best = other > best ? other : best;
+  }
+  if ((threadIdx.x & 63) == 0) s_best[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kSampleThreads / 64; ++w) best = s_best[w] > best ? s_best[w] : best;
+    out[blockIdx.x] = static_cast<int64_t>(~static_cast<uint32_t>(best & 0xFFFFFFFFull));
+  }
+}
+
 }  // namespace
 }  // namespace e2h
+
+extern "C" int e2h_argmax_rows(const uint16_t *logits, int64_t row_stride, int64_t *idx, int64_t rows, int64_t vocab, void *stream) {
+  using namespace e2h;
+  if (!logits || !idx) return E2H_ERR_NULL_POINTER;
+  if (rows < 1 || vocab < 1 || rows > INT32_MAX || vocab > INT32_MAX || row_stride < vocab) return E2H_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(logits) & 1u) || (reinterpret_cast<uintptr_t>(idx) & 7u)) return E2H_ERR_MISALIGNED;
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(static_cast<unsigned>(rows)), dim3(kSampleThreads), 0, static_cast<hipStream_t>(stream), logits,
+                     row_stride, idx, static_cast<int>(vocab));
+  return launch_status();
+}
 
 extern "C" int e2h_sample_top_k(const uint16_t *logits, int64_t row_stride, const float *q, float *probs, int32_t *idx,
                                 int64_t rows, int64_t vocab, float temperature, int top_k, void *stream) {

@@ -18,7 +18,10 @@ from . import ops
 
 def greedy_token(logits: Tensor) -> Tensor:
     """argmax over the vocabulary of the last position, in float32 -> [B, 1] int64."""
-    return torch.argmax(logits[:, -1].float(), dim=-1, keepdim=True)
+    last = logits[:, -1]
+    if last.is_cuda and last.dtype == torch.bfloat16 and not torch.compiler.is_compiling():
+        return ops.argmax_rows(last)
+    return torch.argmax(last.float(), dim=-1, keepdim=True)
 
 
 def multinomial_sample_one_no_sync(probs_sort: Tensor) -> Tensor:

@@ -470,6 +470,20 @@ def sample_top_k(logits, q, temperature=1.0, top_k=None):
     return idx, probs
 
 
+def argmax_rows(logits):
+    """logits bf16 [B, V] (rows may be strided) -> int64 [B, 1]: torch.argmax(logits.float(), dim=-1, keepdim=True) in one launch
+    (lowest index among ties, a NaN counts as the maximum)."""
+    _need_gpu(logits)
+    assert logits.dtype == torch.bfloat16 and logits.dim() == 2
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    rows, vocab = logits.shape
+    idx = torch.empty((rows, 1), dtype=torch.int64, device=logits.device)
+    rc = _lib_for(logits).e2h_argmax_rows(_ptr(logits), logits.stride(0), _ptr(idx), rows, vocab, _stream(logits))
+    _lib.check(rc, "e2h_argmax_rows")
+    return idx
+
+
 def decode_attention(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, scale=None):
     """q bf16 [B, H, D] against caches [Bmax, Hkv, S, D] up to and including input_pos -> bf16 [B, H, D]."""
     _need_gpu(q, k_cache, v_cache, input_pos)

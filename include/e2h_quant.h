@@ -214,6 +214,12 @@ int e2h_silu_mul(const uint16_t *a, const uint16_t *b, uint16_t *y, int64_t n, v
 int e2h_sample_top_k(const uint16_t *logits, int64_t row_stride, const float *q, float *probs, int32_t *idx,
                      int64_t rows, int64_t vocab, float temperature, int top_k, void *stream);
 
+/* Greedy next token: idx[r] = argmax(float(logits[r, :])) (the harness's temperature-free path; the reference's
+ * torch.argmax over the last position's logits, inference_generate.py:110-120 with sampling switched off).
+ *   logits bf16, row r starts at logits + r * row_stride (row_stride >= vocab, in elements); idx int64 [rows].
+ * Ties go to the lowest index; a NaN counts as the largest value (ATen's arg-max convention). */
+int e2h_argmax_rows(const uint16_t *logits, int64_t row_stride, int64_t *idx, int64_t rows, int64_t vocab, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

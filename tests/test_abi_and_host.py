@@ -202,6 +202,9 @@ def test_fused_and_sampling_entry_points_validate_arguments():
     assert lib.e2h_sample_top_k(p, 10, p, p, p, 2, 16, 1.0, 0, None) == -2
     assert lib.e2h_sample_top_k(p, 16, p, p, p, 2, 16, 1.0, -1, None) == -2
     assert lib.e2h_sample_top_k(p, 16, ctypes.c_void_p(4098), p, p, 2, 16, 1.0, 0, None) == -5
+    assert lib.e2h_argmax_rows(p, 10, p, 2, 16, None) == -2
+    assert lib.e2h_argmax_rows(p, 16, null, 2, 16, None) == -1
+    assert lib.e2h_argmax_rows(p, 16, ctypes.c_void_p(4100), 2, 16, None) == -5
     for name in (b"row_tiles", b"int4_no_xsum", b"int4_no_gemm32", b"int4_gemm32_min_rows"):
         assert lib.e2h_set_option(name, 0) == 0
     assert lib.e2h_set_option(b"row_tiles", 3) == -8

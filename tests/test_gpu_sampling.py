@@ -51,6 +51,26 @@ def test_sample_strided_rows_and_top1_is_argmax():
     assert torch.all((probs > 0).sum(-1) >= 1)
 
 
+@pytest.mark.parametrize("rows,vocab", [(1, 512), (32, 32000), (5, 32016), (3, 1001), (2, 7)])
+def test_argmax_rows_is_torch_argmax_with_ties_and_nan(rows, vocab):
+    """Greedy choice: bit-for-bit torch.argmax(logits.float()) -- bfloat16 logits tie often, ties must go to the lowest
+    index -- on contiguous rows, strided rows (the [:, -1] view of [B, S, V] logits) and a row containing a NaN."""
+    gen = torch.Generator().manual_seed(rows + vocab)
+    full = (torch.randn((rows, 2, vocab), generator=gen) * 2.0).to(torch.bfloat16)
+    full[0, -1, vocab // 2] = full[0, -1].float().max()  # an exact tie with the maximum somewhere earlier or later
+    full = full.to(DEV)
+    for logits in (full[:, -1], full[:, -1].contiguous(), full[:, 0]):
+        idx = ops.argmax_rows(logits)
+        assert idx.dtype == torch.int64 and idx.shape == (rows, 1)
+        ref_val = logits.float().max(-1, keepdim=True).values
+        assert torch.equal(logits.float().gather(1, idx), ref_val)
+        first = (logits.float() == ref_val).float().argmax(-1, keepdim=True)  # lowest index attaining the maximum
+        assert torch.equal(idx, first)
+    nan_row = full[:, -1].contiguous()
+    nan_row[-1, vocab - 1] = float("nan")
+    assert int(ops.argmax_rows(nan_row)[-1, 0]) == vocab - 1
+
+
 def test_sampling_frequencies_follow_probs():
     """Exponential race = multinomial sampling: empirical frequencies of 20000 draws match probs (chi-square-ish bound)."""
     torch.manual_seed(0)
