@@ -36,6 +36,8 @@ _SIGNATURES = {
     "e2h_int4_mm_rope_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, _P]),
     "e2h_sample_top_k": (c_int, [_P, c_int64, _P, _P, _P, c_int64, c_int64, c_float, c_int, _P]),
     "e2h_argmax_rows": (c_int, [_P, c_int64, _P, c_int64, c_int64, _P]),
+    "e2h_int8_mm_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, _P]),
+    "e2h_int8_mm_rope_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
     "e2h_int4_mm_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P]),
 }
 

@@ -48,11 +48,33 @@ struct WeightRegs8 {
   u32x4_t w[T][2];
 };
 
-template <int MT, int T, int WN, int WK>
+// Epilogues of the decode step (one launch each, at most 64 rows, no K split over workgroups):
+// kGate8: the wave's two tiles are the same 16 columns of two weight matrices (q / scales and q2 / scales2, the gate
+//   and up projections of a feed-forward block); stores bf16(bf16(silu(g)) * u) with g, u the two linears' bfloat16
+//   outputs -- the rounding points of F.silu(w1(x)) * w3(x) on bfloat16 tensors (reference models/model.py:343-344).
+// kRope8: the product is the fused q | k | v projection of ONE new token per sequence (row m = sequence m); the
+//   bfloat16 output is rotated in float32 by the angle of position input_pos[0] (interleaved pairs, reference
+//   models/model.py:400-412); q goes to q_out [B, H, D], k and v into the caches [B, Hkv, S, D] at that position
+//   (KVCache.update, reference models/model.py:94-104).
+enum Epilogue8 { kPlain8 = 0, kGate8 = 1, kRope8 = 2 };
+
+struct Rope8Args {
+  const uint16_t *freqs;     // [>= S, D/2, 2] bf16 (cos, sin)
+  uint16_t *q_out, *kc, *vc;
+  const int64_t *input_pos;  // [1] on the device
+  int H, Hkv, S, D;
+};
+
+template <int MT, int T, int WN, int WK, int EPI = kPlain8>
 __global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
-                                                                      const uint16_t *__restrict__ scales, uint16_t *__restrict__ y,
+                                                                      const uint16_t *__restrict__ scales, const int8_t *__restrict__ q2,
+                                                                      const uint16_t *__restrict__ scales2, uint16_t *__restrict__ y,
                                                                       float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket,
-                                                                      int M, int N, int K) {
+                                                                      int M, int N, int K, Rope8Args rope) {
+  constexpr bool GATE = EPI == kGate8;
+  static_assert(!GATE || T == 2, "gate mode pairs exactly two weight matrices");
+  static_assert(EPI != kRope8 || T == 1, "the rotary epilogue handles one column tile per wave");
+  constexpr int TC = GATE ? 1 : T;  // distinct column tiles per wave
   typedef Tuning8<MT, T, WN, WK> Tune;
   constexpr int NB = Tune::NB, PD = NB - 1, CPP = Tune::CPP, XD = Tune::XD;
   constexpr int U = NB > CPP * XD ? NB : CPP * XD;
@@ -87,26 +109,28 @@ __global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint
   const int c1 = C0 + ((C1 - C0) * (kg + 1)) / WK;
   const int nloc = c1 - c0;
   const int nloc_max = (C1 - C0 + WK - 1) / WK;
-  const int tile16_0 = (blockIdx.x * WN + wave_n) * T;
+  const int tile16_0 = (blockIdx.x * WN + wave_n) * TC;
   const int m_base = blockIdx.z * (16 * MT);
   uint8_t *const xlds = lds + kg * (2 * kStageBytes);
 
   uint32_t wlane[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) {
-    int n = 16 * (tile16_0 + t) + c;
+    int n = 16 * (tile16_0 + (GATE ? 0 : t)) + c;
     n = n < N ? n : N - 1;
     wlane[t] = static_cast<uint32_t>(static_cast<size_t>(n) * K + 16 * b);
   }
   const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(q, static_cast<uint32_t>(static_cast<size_t>(N) * K));
+  const __amdgpu_buffer_rsrc_t w2_rsrc = make_rsrc(GATE ? q2 : q, static_cast<uint32_t>(static_cast<size_t>(N) * K));
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
 
   auto load_weights = [&](WeightRegs8<T> &r, int ci) {
     const uint32_t so = static_cast<uint32_t>(ci) * kChunk;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      r.w[t][0] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[t], so, 2);
-      r.w[t][1] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wlane[t], so + 64, 2);
+      const __amdgpu_buffer_rsrc_t wr = (GATE && t == 1) ? w2_rsrc : w_rsrc;
+      r.w[t][0] = __builtin_amdgcn_raw_buffer_load_b128(wr, wlane[t], so, 2);
+      r.w[t][1] = __builtin_amdgcn_raw_buffer_load_b128(wr, wlane[t], so + 64, 2);
     }
   };
 
@@ -178,11 +202,24 @@ __global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint
 
   WeightRegs8<T> ring[NB];
   u32x4_t xstage[XD][kPiecesPerThread];
+  int rope_pos = -1;
+  float rope_cs = 1.f, rope_sn = 0.f;
   if (C1 > C0) {
 #pragma unroll
     for (int d = 0; d < XD; ++d) load_x(xstage[d], d);
 #pragma unroll
     for (int i = 0; i < PD; ++i) load_weights(ring[i], chunk_at(i));
+    if constexpr (EPI == kRope8) {
+      // cos / sin depend on a position read from memory: fetch both behind the first weight loads instead of as two
+      // dependent round trips at the very end
+      rope_pos = static_cast<int>(rope.input_pos[0]);
+      const int ncol = 16 * tile16_0 + c;
+      if (ncol < N && rope_pos >= 0 && rope_pos < rope.S && ncol < (rope.H + rope.Hkv) * rope.D) {
+        const uint32_t f = reinterpret_cast<const uint32_t *>(rope.freqs)[static_cast<size_t>(rope_pos) * (rope.D / 2) + ((ncol % rope.D) >> 1)];
+        rope_cs = __builtin_bit_cast(float, f << 16);
+        rope_sn = __builtin_bit_cast(float, f & 0xFFFF0000u);
+      }
+    }
     store_x(xstage[0], 0);
     lds_barrier();
     for (int base = 0; base < nloc_max; base += U) {
@@ -267,6 +304,51 @@ __global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint
     }
   }
   if (kg != 0) return;
+  if constexpr (EPI == kRope8) {
+    const int n = 16 * tile16_0 + c;
+    const float scale = bf16_to_f32(scales[n < N ? n : N - 1]);
+    const int D = rope.D, H = rope.H, Hkv = rope.Hkv;
+    const int head = n / D, d = n % D;
+    const int pos = rope_pos;
+    const bool in_range = n < N && pos >= 0 && pos < rope.S;
+    const bool rotated = head < H + Hkv;
+    uint16_t *dst;  // element (m = 0) of this lane's column; rows are row_stride apart
+    size_t row_stride;
+    if (head < H) {
+      dst = rope.q_out + static_cast<size_t>(head) * D + d;
+      row_stride = static_cast<size_t>(H) * D;
+    } else {
+      const int hk = rotated ? head - H : head - H - Hkv;
+      dst = (rotated ? rope.kc : rope.vc) + (static_cast<size_t>(hk) * rope.S + pos) * D + d;
+      row_stride = static_cast<size_t>(Hkv) * rope.S * D;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m_base + 16 * mt + 4 * b + r;
+        const float own = bf16_round(bf16_round(acc[0][mt][r]) * scale);  // the linear's bfloat16 output
+        const float other = __shfl_xor(own, 1);                           // the pair's other column lives in the neighbouring lane
+        // even column: x0 * cos - x1 * sin; odd column: x1 * cos + x0 * sin (two rounded products, then the sum)
+        const float rot = (c & 1) ? own * rope_cs + other * rope_sn : own * rope_cs - other * rope_sn;
+        if (in_range && m < M) dst[static_cast<size_t>(m) * row_stride] = f32_to_bf16_rne(rotated ? rot : own);
+      }
+    return;
+  }
+  if constexpr (GATE) {
+    const int n = 16 * tile16_0 + c;
+    const float s_gate = bf16_to_f32(scales[n < N ? n : N - 1]), s_up = bf16_to_f32(scales2[n < N ? n : N - 1]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m_base + 16 * mt + 4 * b + r;
+        const float gate = bf16_round(bf16_round(acc[0][mt][r]) * s_gate), up = bf16_round(bf16_round(acc[1][mt][r]) * s_up);
+        const float act = bf16_round(gate / (1.0f + expf(-gate)));
+        if (n < N && m < M) y[static_cast<size_t>(m) * N + n] = f32_to_bf16_rne(act * up);
+      }
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const int n = 16 * (tile16_0 + t) + c;
@@ -288,6 +370,9 @@ struct Args8 {
   const uint16_t *x;
   const int8_t *q;
   const uint16_t *scales;
+  const int8_t *q2 = nullptr;       // second weight matrix of the gated form
+  const uint16_t *scales2 = nullptr;
+  Rope8Args rope = {};
   uint16_t *y;
   float *ws_partial;
   unsigned *ws_ticket;
@@ -295,12 +380,13 @@ struct Args8 {
   hipStream_t stream;
 };
 
-template <int MT, int T, int WN, int WK>
+template <int MT, int T, int WN, int WK, int EPI = kPlain8>
 int launch8(const Args8 &a) {
   const int tiles16 = (a.N + 15) / 16;
-  dim3 grid((tiles16 + WN * T - 1) / (WN * T), a.S, (a.M + 16 * MT - 1) / (16 * MT));
-  hipLaunchKernelGGL((int8_stream_mm_kernel<MT, T, WN, WK>), grid, dim3(64 * WN * WK), 0, a.stream, a.x, a.q, a.scales, a.y,
-                     a.ws_partial, a.ws_ticket, a.M, a.N, a.K);
+  constexpr int TC = EPI == kGate8 ? 1 : T;
+  dim3 grid((tiles16 + WN * TC - 1) / (WN * TC), a.S, (a.M + 16 * MT - 1) / (16 * MT));
+  hipLaunchKernelGGL((int8_stream_mm_kernel<MT, T, WN, WK, EPI>), grid, dim3(64 * WN * WK), 0, a.stream, a.x, a.q, a.scales, a.q2,
+                     a.scales2, a.y, a.ws_partial, a.ws_ticket, a.M, a.N, a.K, a.rope);
   return launch_status();
 }
 
@@ -377,3 +463,42 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
 }
 
 }  // namespace e2h
+
+extern "C" int e2h_int8_mm_silu_gate(const uint16_t *x, const int8_t *q_gate, const uint16_t *scales_gate, const int8_t *q_up,
+                                     const uint16_t *scales_up, uint16_t *y, int64_t m, int64_t n, int64_t k, void *stream) {
+  using namespace e2h;
+  if (!x || !q_gate || !scales_gate || !q_up || !scales_up || !y) return E2H_ERR_NULL_POINTER;
+  if (m < 1 || m > 64 || n < 1 || k < 128 || (k % 128) != 0 || n > INT32_MAX || k > INT32_MAX || n * k >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(q_gate) || !aligned16(q_up) || (reinterpret_cast<uintptr_t>(scales_gate) & 1u) ||
+      (reinterpret_cast<uintptr_t>(scales_up) & 1u) || (reinterpret_cast<uintptr_t>(y) & 1u))
+    return E2H_ERR_MISALIGNED;
+  Args8 a;
+  a.x = x; a.q = q_gate; a.scales = scales_gate; a.q2 = q_up; a.scales2 = scales_up; a.y = y;
+  a.ws_partial = nullptr; a.ws_ticket = nullptr;
+  a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k); a.S = 1;
+  a.stream = static_cast<hipStream_t>(stream);
+  return a.M <= 16 ? launch8<1, 2, 4, 2, kGate8>(a) : launch8<2, 2, 4, 2, kGate8>(a);
+}
+
+extern "C" int e2h_int8_mm_rope_kv(const uint16_t *x, const int8_t *q, const uint16_t *scales, const uint16_t *freqs_cis, uint16_t *q_out,
+                                   uint16_t *k_cache, uint16_t *v_cache, const int64_t *input_pos, int64_t batch, int64_t n_head,
+                                   int64_t n_kv_head, int64_t head_dim, int64_t cache_len, int64_t k, void *stream) {
+  using namespace e2h;
+  if (!x || !q || !scales || !freqs_cis || !q_out || !k_cache || !v_cache || !input_pos) return E2H_ERR_NULL_POINTER;
+  if (batch < 1 || batch > 64 || n_head < 1 || n_kv_head < 1 || head_dim < 2 || (head_dim % 2) != 0 || cache_len < 1 || k < 128 || (k % 128) != 0)
+    return E2H_ERR_BAD_SHAPE;
+  const int64_t n = (n_head + 2 * n_kv_head) * head_dim;
+  if (n > INT32_MAX || k > INT32_MAX || cache_len > INT32_MAX || n * k >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(q) || (reinterpret_cast<uintptr_t>(scales) & 1u) || (reinterpret_cast<uintptr_t>(freqs_cis) & 3u) ||
+      (reinterpret_cast<uintptr_t>(q_out) & 1u) || (reinterpret_cast<uintptr_t>(k_cache) & 1u) || (reinterpret_cast<uintptr_t>(v_cache) & 1u) ||
+      (reinterpret_cast<uintptr_t>(input_pos) & 7u))
+    return E2H_ERR_MISALIGNED;
+  Args8 a;
+  a.x = x; a.q = q; a.scales = scales; a.y = nullptr;
+  a.rope = Rope8Args{freqs_cis, q_out, k_cache, v_cache, input_pos, static_cast<int>(n_head), static_cast<int>(n_kv_head),
+                     static_cast<int>(cache_len), static_cast<int>(head_dim)};
+  a.ws_partial = nullptr; a.ws_ticket = nullptr;
+  a.M = static_cast<int>(batch); a.N = static_cast<int>(n); a.K = static_cast<int>(k); a.S = 1;
+  a.stream = static_cast<hipStream_t>(stream);
+  return a.M <= 16 ? launch8<1, 1, 4, 2, kRope8>(a) : launch8<2, 1, 4, 2, kRope8>(a);
+}

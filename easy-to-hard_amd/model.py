@@ -16,7 +16,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from . import ops
-from .quantize import WeightOnlyInt4Linear, find_multiple
+from .quantize import WeightOnlyInt4Linear, WeightOnlyInt8Linear, find_multiple
 
 # When True (default) and the tensors are bf16 on the GPU, RMSNorm, SiLU*mul and -- for single-token steps with
 # a KV cache -- RoPE + cache write + attention run as this package's fused kernels instead of chains of stock ops.
@@ -179,6 +179,9 @@ class Attention(nn.Module):
                 q = ops.int4_mm_rope_kv(x.view(bsz, -1), w.weight, w.scales_and_zeros, w.groupsize, self.freqs_table,
                                         self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, self.n_head,
                                         self.n_local_heads, self.head_dim)
+            elif FUSE_ROPE_PROJECTION and isinstance(w, WeightOnlyInt8Linear) and ops.int8_rope_kv_supported(x, w, self.freqs_table, self.kv_cache.k_cache):
+                q = ops.int8_mm_rope_kv(x.view(bsz, -1), w.weight, w.scales, self.freqs_table, self.kv_cache.k_cache,
+                                        self.kv_cache.v_cache, input_pos, self.n_head, self.n_local_heads, self.head_dim)
             else:
                 qkv = w(x).view(bsz, -1)
                 q = ops.rope_kv_write(qkv, self.freqs_table, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos,
@@ -231,7 +234,16 @@ class FeedForward(nn.Module):
             return False
         return ops.int4_gate_supported(x, w1, w3)
 
+    def _gate_fusable_int8(self, x: Tensor) -> bool:
+        w1, w3 = self.w1, self.w3
+        if not (FUSED_DECODE and FUSE_GATE and isinstance(w1, WeightOnlyInt8Linear) and isinstance(w3, WeightOnlyInt8Linear)):
+            return False
+        return not torch.compiler.is_compiling() and ops.int8_gate_supported(x, w1, w3)
+
     def forward(self, x: Tensor) -> Tensor:
+        if self._gate_fusable_int8(x):
+            y = ops.int8_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales, self.w3.weight, self.w3.scales)
+            return self.w2(y.reshape(*x.shape[:-1], y.shape[-1]))
         if self._gate_fusable(x):
             # silu(w1 x) * w3 x in one launch: both products share the activation stream
             y = ops.int4_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales_and_zeros,

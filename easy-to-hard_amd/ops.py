@@ -452,6 +452,67 @@ def int4_mm_rope_kv(x, packed, scales_and_zeros, groupsize, freqs_cis, k_cache, 
     return q
 
 
+def _int8_fusable(x, *mods):
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() // x.shape[-1] <= 64 and x.shape[-1] % 128 == 0):
+        return False
+    for m in mods:
+        if m.weight.dtype != torch.int8 or m.weight.dim() != 2 or m.scales.dtype != torch.bfloat16 or m.weight.shape[1] != x.shape[-1]:
+            return False
+        if m.weight.shape[0] * m.weight.shape[1] >= 2 ** 32:
+            return False
+    return True
+
+
+def int8_gate_supported(x, w_gate, w_up):
+    """True when (x, two WeightOnlyInt8Linear modules) fit e2h_int8_mm_silu_gate's contract."""
+    return _int8_fusable(x, w_gate, w_up) and w_gate.weight.shape == w_up.weight.shape
+
+
+def int8_mm_silu_gate(x, q_gate, scales_gate, q_up, scales_up):
+    """bf16(bf16(silu(int8_mm(x, gate))) * int8_mm(x, up)) in one launch; x bf16 [M <= 64, K]."""
+    _need_gpu(x, q_gate, scales_gate, q_up, scales_up)
+    assert x.dtype == torch.bfloat16 and x.dim() == 2 and q_gate.dtype == torch.int8 and q_up.dtype == torch.int8
+    assert scales_gate.dtype == torch.bfloat16 and scales_up.dtype == torch.bfloat16
+    n, k = q_gate.shape
+    if q_up.shape != q_gate.shape or x.shape[1] != k or scales_gate.numel() != n or scales_up.numel() != n:
+        raise RuntimeError("int8_mm_silu_gate: shapes of the two linears and x do not match")
+    x, q_gate, q_up = x.contiguous(), q_gate.contiguous(), q_up.contiguous()
+    scales_gate, scales_up = scales_gate.contiguous(), scales_up.contiguous()
+    y = torch.empty((x.shape[0], n), dtype=torch.bfloat16, device=x.device)
+    rc = _lib_for(x).e2h_int8_mm_silu_gate(_ptr(x), _ptr(q_gate), _ptr(scales_gate), _ptr(q_up), _ptr(scales_up), _ptr(y), x.shape[0], n, k,
+                                           _stream(x))
+    _lib.check(rc, "e2h_int8_mm_silu_gate")
+    return y
+
+
+def int8_rope_kv_supported(x, wqkv, freqs_cis, k_cache):
+    """True when the fused projection + RoPE + cache write covers (x [B, 1, K], a WeightOnlyInt8Linear)."""
+    return _int8_fusable(x, wqkv) and freqs_cis.shape[0] >= k_cache.shape[2]
+
+
+def int8_mm_rope_kv(x, q_weight, scales, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head, head_dim):
+    """x bf16 [B <= 64, K] (one new token per sequence) times the int8 fused q|k|v weight, then RoPE and the cache write
+    of rope_kv_write, in one launch.  Returns the rotated q [B, H, D]."""
+    _need_gpu(x, q_weight, scales, freqs_cis, k_cache, v_cache, input_pos)
+    assert x.dtype == torch.bfloat16 and q_weight.dtype == torch.int8 and scales.dtype == torch.bfloat16 and freqs_cis.dtype == torch.bfloat16
+    assert input_pos.dtype == torch.int64 and input_pos.numel() >= 1 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and freqs_cis.is_contiguous() and x.dim() == 2
+    n, k = q_weight.shape
+    bsz = x.shape[0]
+    if n != (n_head + 2 * n_kv_head) * head_dim or x.shape[1] != k or scales.numel() != n:
+        raise RuntimeError(f"int8_mm_rope_kv: weight is [{n}, {k}], expected [{(n_head + 2 * n_kv_head) * head_dim}, {x.shape[1]}]")
+    if k_cache.shape[0] < bsz or k_cache.shape[1] != n_kv_head or k_cache.shape[3] != head_dim or v_cache.shape != k_cache.shape:
+        raise RuntimeError("int8_mm_rope_kv: caches must be [>= B, Hkv, S, D]")
+    if freqs_cis.shape[0] < k_cache.shape[2] or tuple(freqs_cis.shape[1:]) != (head_dim // 2, 2):
+        raise RuntimeError("int8_mm_rope_kv: freqs_cis must be [>= S, D/2, 2]")
+    x, q_weight, scales = x.contiguous(), q_weight.contiguous(), scales.contiguous()
+    q = torch.empty((bsz, n_head, head_dim), dtype=torch.bfloat16, device=x.device)
+    rc = _lib_for(x).e2h_int8_mm_rope_kv(_ptr(x), _ptr(q_weight), _ptr(scales), _ptr(freqs_cis), _ptr(q), _ptr(k_cache), _ptr(v_cache),
+                                         _ptr(input_pos), bsz, n_head, n_kv_head, head_dim, k_cache.shape[2], k, _stream(x))
+    _lib.check(rc, "e2h_int8_mm_rope_kv")
+    return q
+
+
 def sample_top_k(logits, q, temperature=1.0, top_k=None):
     """logits bf16 [B, V] (rows may be strided), q float32 [B, V] of Exp(1) draws -> (idx int32 [B, 1], probs float32 [B, V]):
     softmax(top-k-masked logits / max(temperature, 1e-5)) and argmax(probs / q), in one launch."""

@@ -156,6 +156,18 @@ int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, const uint16_t
                         int64_t head_dim, int64_t cache_len, int64_t k, int groupsize, int inner_k_tiles,
                         void *stream);
 
+/* int8 forms of the two fused decode-step launches above (WeightOnlyInt8Linear modules, reference
+ * models/quantize.py:405-429, in FeedForward.forward models/model.py:343-344 and Attention.forward :283-296).
+ * Each linear's output is formed with the reference's two roundings, bf16(bf16(x @ q^T) * scales), before the SiLU-gate
+ * or the rotation is applied, so the results equal the unfused sequence of calls bit for bit.
+ *   q_* int8 [n, k] row-major, scales_* bf16 [n]; 1 <= m (batch) <= 64, k % 128 == 0, 16-byte aligned x and q rows;
+ *   the other arguments as in e2h_int4_mm_silu_gate / e2h_int4_mm_rope_kv. */
+int e2h_int8_mm_silu_gate(const uint16_t *x, const int8_t *q_gate, const uint16_t *scales_gate, const int8_t *q_up,
+                          const uint16_t *scales_up, uint16_t *y, int64_t m, int64_t n, int64_t k, void *stream);
+int e2h_int8_mm_rope_kv(const uint16_t *x, const int8_t *q, const uint16_t *scales, const uint16_t *freqs_cis, uint16_t *q_out,
+                        uint16_t *k_cache, uint16_t *v_cache, const int64_t *input_pos, int64_t batch, int64_t n_head,
+                        int64_t n_kv_head, int64_t head_dim, int64_t cache_len, int64_t k, void *stream);
+
 /* Recommended size in bytes of the workspace accepted by the matmul entry points (no reference counterpart). */
 int64_t e2h_workspace_bytes(void);
 

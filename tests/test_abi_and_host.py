@@ -202,6 +202,12 @@ def test_fused_and_sampling_entry_points_validate_arguments():
     assert lib.e2h_sample_top_k(p, 10, p, p, p, 2, 16, 1.0, 0, None) == -2
     assert lib.e2h_sample_top_k(p, 16, p, p, p, 2, 16, 1.0, -1, None) == -2
     assert lib.e2h_sample_top_k(p, 16, ctypes.c_void_p(4098), p, p, 2, 16, 1.0, 0, None) == -5
+    # int8 fused launches: too many rows, K not in whole chunks, null pointer
+    assert lib.e2h_int8_mm_silu_gate(p, p, p, p, p, p, 65, 64, 128, None) == -2
+    assert lib.e2h_int8_mm_silu_gate(p, p, p, p, p, p, 32, 64, 192, None) == -2
+    assert lib.e2h_int8_mm_silu_gate(p, null, p, p, p, p, 32, 64, 128, None) == -1
+    assert lib.e2h_int8_mm_rope_kv(p, p, p, p, p, p, p, p, 4, 2, 2, 63, 16, 128, None) == -2
+    assert lib.e2h_int8_mm_rope_kv(p, p, p, p, p, p, p, null, 4, 2, 2, 64, 16, 128, None) == -1
     assert lib.e2h_argmax_rows(p, 10, p, 2, 16, None) == -2
     assert lib.e2h_argmax_rows(p, 16, null, 2, 16, None) == -1
     assert lib.e2h_argmax_rows(p, 16, ctypes.c_void_p(4100), 2, 16, None) == -5

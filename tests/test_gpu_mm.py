@@ -455,3 +455,63 @@ def test_int4_mm_matches_the_stock_rocm_op_on_identical_codes(m):
         pytest.skip(f"stock aten._weight_int4pack_mm unavailable here: {exc}")
     y = ops.int4_mm_direct(x, packed, g, sz).float()
     assert float((y - y_stock).abs().max() / y_stock.abs().max()) <= 1e-2
+
+
+# ---- int8 forms of the two fused decode-step launches ----
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("n,k", [(48, 512), (690, 1024), (11008, 4096)])
+def test_int8_gate_matches_oracle_and_unfused_path(m, n, k):
+    if n * k > 1 << 22 and m not in (1, 32, 64):
+        pytest.skip("large shape: three batch sizes only")
+    q1, s1, q1_d, s1_d = _int8_case(n, k, seed=n + m)
+    q2, s2, q2_d, s2_d = _int8_case(n, k, seed=n + m + 7)
+    x = randn_bf16((m, k), std=1.0, seed=m * 31)
+    xd = x.to(DEV)
+    y = ops.int8_mm_silu_gate(xd, q1_d, s1_d, q2_d, s2_d)
+    assert y.dtype == torch.bfloat16 and y.shape == (m, n)
+    a = qo.int8_linear_fp32(bf16_to_np(x), q1, s1).astype(np.float64)
+    b = qo.int8_linear_fp32(bf16_to_np(x), q2, s2).astype(np.float64)
+    assert qo.normwise_rel_err(bf16_to_np(y), a / (1.0 + np.exp(-a)) * b) <= TOL
+    # same accumulation order as the single-matrix kernel with one K slice: identical bits
+    _lib.set_option("int8_k_slices", 1)
+    try:
+        ya = ops.int8_mm_direct(xd, q1_d, s1_d)
+        yb = ops.int8_mm_direct(xd, q2_d, s2_d)
+    finally:
+        _lib.set_option("int8_k_slices", 0)
+    assert torch.equal(y, ops.silu_mul(ya, yb) if (m * n) % 8 == 0 else torch.nn.functional.silu(ya) * yb)
+    with pytest.raises(RuntimeError):
+        ops.int8_mm_silu_gate(randn_bf16((65, k), seed=3).to(DEV), q1_d, s1_d, q2_d, s2_d)  # more than 64 rows
+
+
+@pytest.mark.parametrize("bsz", [1, 3, 16, 32, 40, 64])
+@pytest.mark.parametrize("n_head,n_kv,d,k", [(4, 4, 64, 256), (8, 2, 64, 512), (32, 32, 128, 4096), (6, 3, 128, 384)])
+def test_int8_rope_kv_matches_two_kernel_path(bsz, n_head, n_kv, d, k):
+    from easy_to_hard_amd.model import precompute_freqs_cis
+
+    if k == 4096 and bsz not in (1, 32, 64):
+        pytest.skip("large shape: three batch sizes only")
+    n = (n_head + 2 * n_kv) * d
+    s_max, pos = 80, 37
+    _, _, q_d, s_d = _int8_case(n, k, seed=n + bsz)
+    x = randn_bf16((bsz, k), std=1.0, seed=bsz * 17).to(DEV)
+    gen = torch.Generator().manual_seed(n_head + d)
+    kc0 = torch.randn((bsz + 1, n_kv, s_max, d), generator=gen).to(torch.bfloat16).to(DEV)
+    vc0 = torch.randn((bsz + 1, n_kv, s_max, d), generator=gen).to(torch.bfloat16).to(DEV)
+    freqs = precompute_freqs_cis(s_max, d, 10000, device=DEV)
+    input_pos = torch.tensor([pos], device=DEV)
+    kc, vc = kc0.clone(), vc0.clone()
+    q = ops.int8_mm_rope_kv(x, q_d, s_d, freqs, kc, vc, input_pos, n_head, n_kv, d)
+    _lib.set_option("int8_k_slices", 1)
+    try:
+        qkv = ops.int8_mm_direct(x, q_d, s_d)
+    finally:
+        _lib.set_option("int8_k_slices", 0)
+    kc2, vc2 = kc0.clone(), vc0.clone()
+    q2 = ops.rope_kv_write(qkv, freqs, kc2, vc2, input_pos, n_head, n_kv, d)
+    assert torch.equal(q, q2) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    # a position outside the cache writes nothing
+    kc3, vc3 = kc0.clone(), vc0.clone()
+    ops.int8_mm_rope_kv(x, q_d, s_d, freqs, kc3, vc3, torch.tensor([s_max], device=DEV), n_head, n_kv, d)
+    assert torch.equal(kc3, kc0) and torch.equal(vc3, vc0)
