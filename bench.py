@@ -103,13 +103,17 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
         parent_name, _, leaf = name.rpartition(".")
         parent = model.get_submodule(parent_name) if parent_name else model
         x = xs[mod.in_features]
-        fused = isinstance(parent, e2h_model.FeedForward) and parent._gate_fusable(x)
+        fused8 = isinstance(parent, e2h_model.FeedForward) and parent._gate_fusable_int8(x)
+        fused = fused8 or (isinstance(parent, e2h_model.FeedForward) and parent._gate_fusable(x))
         if fused and leaf == "w3":
             continue
         if fused and leaf == "w1":
             up = by_name[parent_name + ".w3"]
-            calls.append(lambda x=x, g=mod, u=up: ops.int4_mm_silu_gate(
-                x, g.weight, g.scales_and_zeros, u.weight, u.scales_and_zeros, g.groupsize))
+            if fused8:
+                calls.append(lambda x=x, g=mod, u=up: ops.int8_mm_silu_gate(x, g.weight, g.scales, u.weight, u.scales))
+            else:
+                calls.append(lambda x=x, g=mod, u=up: ops.int4_mm_silu_gate(
+                    x, g.weight, g.scales_and_zeros, u.weight, u.scales_and_zeros, g.groupsize))
             # two weight matrices, but x is read once and one [batch, n] result is written
             bytes_pass += algorithmic_bytes(mod, batch) + algorithmic_bytes(up, batch) - batch * 2 * (mod.in_features + mod.out_features)
         else:
@@ -150,7 +154,7 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get(traffic_key),
-        "kernel": "int4_skinny_mm_kernel" if "Int4" in type(lins[0][1]).__name__ else "int8_skinny_mm_kernel",
+        "kernel": "int4_skinny_mm_kernel" if "Int4" in type(lins[0][1]).__name__ else "int8_stream_mm_kernel",
         "launches_per_step": len(calls),
         "algorithmic_bytes_per_launch": bytes_pass // len(calls),
         "avg_launch_us": round(avg_launch_s * 1e6, 3),
