@@ -710,6 +710,13 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
   int64_t max_rows = rows_by_bytes < rows_by_grid ? rows_by_bytes : rows_by_grid;
   max_rows -= max_rows % (16 * mt);
   if (max_rows < 16 * mt) return E2H_ERR_BAD_SHAPE;
+  if (mt == 4 && wide_ok && workspace && !options().int4_no_xsum) {
+    // many rows: the pre-pass keeps (K / g) sums per row in the workspace; slice M so that they fit rather than fall
+    // back to the kernels that form the sums themselves (K = 22016 at g = 64: 24k rows per slice with 32 MB)
+    const int64_t avail = workspace_bytes - static_cast<int64_t>(kTicketBytes);
+    const int64_t rows_by_xsum = avail / (static_cast<int64_t>(a.K / groupsize) * 4) / 256 * 256;
+    if (rows_by_xsum >= 2048 && rows_by_xsum < max_rows) max_rows = rows_by_xsum;
+  }
   const int m_total = a.M;
   for (int64_t m0 = 0; m0 < m_total; m0 += max_rows) {
     a.x = x + m0 * a.K;
@@ -794,12 +801,15 @@ extern "C" int e2h_int4_mm_silu_gate(const uint16_t *x, const int32_t *packed_ga
   if (wn < 2 || wn > 4) {
     wn = 4;
     double best = -1.0;
+    const int slabs = (a.M + 16 * mt - 1) / (16 * mt);  // 33 .. 64 rows run as two 32-row slabs of workgroups
     for (int cand = 4; cand >= 2; --cand) {
       if (cand == 3 && groupsize != 128) continue;  // 6-wave workgroups with two tiles and several groups per chunk spill registers
-      const int wgs = (tiles16 + cand - 1) / cand;
+      const int wgs = ((tiles16 + cand - 1) / cand) * slabs;
       const int rounds = (wgs + kCUs - 1) / kCUs;
       const double fill = static_cast<double>(wgs) / (static_cast<double>(rounds) * kCUs);
-      if (fill > best + 0.05) { best = fill; wn = cand; }
+      // four-wave workgroups (one wave per SIMD) hide latency worst: they must fill the chip much better to pay off
+      // (measured on 2 x 22016 x 8192 at 64 rows: 119 us with two column waves, 100 us with four)
+      if (fill > best + (cand == 2 ? 0.25 : 0.05)) { best = fill; wn = cand; }
     }
   }
   switch (groupsize) {
