@@ -92,5 +92,9 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.int8_gemm_tile = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "attention_no_mfma")) {
+    o.attention_no_mfma = value != 0;
+    return E2H_OK;
+  }
   return E2H_ERR_BAD_OPTION;
 }

@@ -178,6 +178,180 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_kernel(const uint16_
 }
 
 // ------------------------------------------------------------------------------------------------
+// decode attention for grouped queries (REP = 4 .. 16 query heads per kv head, head_dim 128) on the matrix cores.
+// With several query heads per K / V row the float32 dot products of the kernel above become the bound (8 heads:
+// 3.5 x slower than the memory traffic allows), so both products go through v_mfma_f32_16x16x32_bf16:
+//   S [heads x positions] = Q K^T:  A = Q (rows = heads, padded to 16; 4 steps of 32 over head_dim), B = K^T -- lane
+//     (b, c) of a B operand is 16 contiguous bytes of K row `position c`, read straight from the cache;
+//   O [heads x head_dim] += P V:    A = P (bfloat16, through a 1 KB wave-private LDS tile that turns the accumulator
+//     layout of S into operand layout), B = V -- contracted over positions, so its operand needs 8 consecutive
+//     positions of one column: the wave's V tile (32 positions) goes through LDS and is gathered from there.
+// One workgroup per (sequence, kv head), waves take tiles of 32 positions round robin, online softmax in float32 on
+// the accumulator layout (lane (c, b) holds positions c / heads 4b .. 4b+3 of S, head_dim column c / the same heads of
+// O); the softmax scale is applied to S in float32, Q stays exact.  Visibility as above.
+// ------------------------------------------------------------------------------------------------
+constexpr int kGqaVRow = 264;  // bytes per V row in LDS (256 + 8: rows 8 apart land 16 banks apart)
+
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
+                                                                       const uint16_t *__restrict__ vc, uint16_t *__restrict__ out,
+                                                                       const int64_t *__restrict__ input_pos,
+                                                                       const int64_t *__restrict__ left_pad, int H, int Hkv, int S, int rep,
+                                                                       float scale) {
+  constexpr int D = 128;
+  constexpr int kWaveLds = 1024 + 32 * kGqaVRow;                  // P tile + V tile
+  constexpr int kLoopLds = NW * kWaveLds;
+  constexpr int kEndLds = NW * (16 * D + 32) * 4;                 // per wave: O [16][D], m [16], l [16] as float32
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kLoopLds > kEndLds ? kLoopLds : kEndLds];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, b = lane >> 4;
+  const int bi = blockIdx.x / Hkv, hk = blockIdx.x % Hkv;
+  const int pos = static_cast<int>(input_pos[0]);
+  const int first = left_pad ? static_cast<int>(left_pad[bi]) : 0;
+  const int n_live = pos + 1 < S ? pos + 1 : S;
+
+  // Q as A operands: lane (b, r) holds Q[head r][32 s + 8 b .. + 7]; rows beyond rep are zero
+  bf16x8_t qa[4];
+#pragma unroll
+  for (int s4 = 0; s4 < 4; ++s4) {
+    u32x4_t raw = {0u, 0u, 0u, 0u};
+    if (c < rep) raw = *reinterpret_cast<const u32x4_t *>(q + (static_cast<size_t>(bi) * H + hk * rep + c) * D + 32 * s4 + 8 * b);
+    qa[s4] = __builtin_bit_cast(bf16x8_t, raw);
+  }
+  const size_t head_base = (static_cast<size_t>(bi) * Hkv + hk) * S * D;
+  const uint16_t *kbase = kc + head_base + 8 * b;  // + position * D + 32 s
+  const uint16_t *vbase = vc + head_base;
+  uint8_t *const p_lds = lds + wave * kWaveLds;
+  uint8_t *const v_lds = p_lds + 1024;
+
+  float m_run[4], l_part[4];
+  f32x4_t oacc[8];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m_run[r] = -1e30f;
+    l_part[r] = 0.f;
+  }
+#pragma unroll
+  for (int nt = 0; nt < 8; ++nt) oacc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int t0 = wave * 32; t0 < n_live; t0 += NW * 32) {
+    // K operands of the two 16-position halves and this lane's share of the V tile (row = lane / 2 + 32-row wrap,
+    // eight 16-byte pieces of its half row), all requested before anything is waited for
+    u32x4_t kf[2][4], vr[8];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int tp = t0 + 16 * j + c;
+      const int tc = tp < n_live ? tp : n_live - 1;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) kf[j][s4] = *reinterpret_cast<const u32x4_t *>(kbase + static_cast<size_t>(tc) * D + 32 * s4);
+    }
+    {
+      const int vrow = lane >> 1, vhalf = lane & 1;
+      const int tp = t0 + vrow;
+      const int tc = tp < n_live ? tp : n_live - 1;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) vr[i] = *reinterpret_cast<const u32x4_t *>(vbase + static_cast<size_t>(tc) * D + 64 * vhalf + 8 * i);
+    }
+    // S = Q K^T for 32 positions
+    f32x4_t sacc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      sacc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4)
+        sacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[s4], __builtin_bit_cast(bf16x8_t, kf[j][s4]), sacc[j], 0, 0, 0);
+    }
+    // the V tile goes to LDS while the softmax is worked out
+    {
+      const int vrow = lane >> 1, vhalf = lane & 1;
+      uint8_t *dst = v_lds + vrow * kGqaVRow + 128 * vhalf;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        *reinterpret_cast<u32x2_t *>(dst + 16 * i) = u32x2_t{vr[i][0], vr[i][1]};
+        *reinterpret_cast<u32x2_t *>(dst + 16 * i + 8) = u32x2_t{vr[i][2], vr[i][3]};
+      }
+    }
+    float pv[2][4], corr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sv[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int tp = t0 + 16 * j + c;
+        const bool visible = tp < n_live && (tp >= first || tp == pos);
+        sv[j] = visible ? sacc[j][r] * scale : -1e30f;
+      }
+      float mx = fmaxf(sv[0], sv[1]);
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off));  // over the 16 positions of this head's lanes
+      const float m_new = fmaxf(m_run[r], mx);
+      corr[r] = __expf(m_run[r] - m_new);
+      m_run[r] = m_new;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) pv[j][r] = sv[j] > -1e29f ? __expf(sv[j] - m_new) : 0.f;
+      l_part[r] = l_part[r] * corr[r] + pv[0][r] + pv[1][r];
+    }
+    // P (bfloat16) -> LDS [head][position], then back as the A operand: lane (b, r) = head r, positions 8b .. 8b+7
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) *reinterpret_cast<uint16_t *>(p_lds + (4 * b + r) * 64 + (16 * j + c) * 2) = f32_to_bf16_rne(pv[j][r]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private tiles: the wave's own writes have landed
+    const bf16x8_t pa = *reinterpret_cast<const bf16x8_t *>(p_lds + c * 64 + b * 16);
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) {
+      // V operand of column tile nt: lane (b, c) = positions 8b .. 8b+7 of column 16 nt + c
+      uint32_t vw[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = *reinterpret_cast<const uint16_t *>(v_lds + (8 * b + 2 * i) * kGqaVRow + (16 * nt + c) * 2);
+        const uint32_t hi = *reinterpret_cast<const uint16_t *>(v_lds + (8 * b + 2 * i + 1) * kGqaVRow + (16 * nt + c) * 2);
+        vw[i] = lo | (hi << 16);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) oacc[nt][r] *= corr[r];
+      oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(bf16x8_t, u32x4_t{vw[0], vw[1], vw[2], vw[3]}), oacc[nt], 0, 0, 0);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next tile overwrites the wave's LDS
+  }
+
+  // combine: sum l over the 16 position lanes of each head, then the waves through LDS
+  __syncthreads();  // every wave is done with its loop tiles: the LDS is reused
+  float *const sh_o = reinterpret_cast<float *>(lds);                 // [NW][16][D]
+  float *const sh_m = sh_o + NW * 16 * D;                             // [NW][16]
+  float *const sh_l = sh_m + NW * 16;                                 // [NW][16]
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float l = l_part[r];
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) l += __shfl_xor(l, off);
+    const int head = 4 * b + r;
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) sh_o[(wave * 16 + head) * D + 16 * nt + c] = oacc[nt][r];
+    if (c == 0) {
+      sh_m[wave * 16 + head] = m_run[r];
+      sh_l[wave * 16 + head] = l;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < rep * D; e += 64 * NW) {
+    const int r = e / D, d = e % D;
+    float m = sh_m[r];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) m = fmaxf(m, sh_m[w * 16 + r]);
+    float l = 0.f, a = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float cw = __expf(sh_m[w * 16 + r] - m);
+      l += sh_l[w * 16 + r] * cw;
+      a += sh_o[(w * 16 + r) * D + d] * cw;
+    }
+    out[(static_cast<size_t>(bi) * H + hk * rep + r) * D + d] = f32_to_bf16_rne(a / l);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // RMSNorm (reference :363-377): bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w), float32 statistics.
 // ------------------------------------------------------------------------------------------------
 // One workgroup of BLOCK threads per row.  With `delta` the kernel first forms h = bf16(x + delta) (the residual add
@@ -368,6 +542,14 @@ template <int D>
 int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
                      const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
   const int nw = options().attention_waves ? options().attention_waves : (S > 256 ? 8 : 4);
+  if (D == 128 && rep >= 4 && rep <= 16 && !options().attention_no_mfma) {
+    // several query heads per K / V row: both products on the matrix cores
+    if (nw == 8)
+      hipLaunchKernelGGL(decode_attention_gqa_kernel<8>, grid, dim3(512), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale);
+    else
+      hipLaunchKernelGGL(decode_attention_gqa_kernel<4>, grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale);
+    return launch_status();
+  }
   if (nw == 8) return launch_attention_nw<D, 8>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale);
   return launch_attention_nw<D, 4>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale);
 }

@@ -48,6 +48,7 @@ struct Options {
   int int4_gemm32_min_rows;  // 0 = by workgroup count, else rows from which the 32x32-tile kernels take over
   int row_tiles;           // 0 = heuristic, else 1/2/4 tiles of 16 activation rows per workgroup (both matmuls)
   int attention_waves;     // 0 = by cache length, else 4 or 8 waves per decode-attention workgroup
+  int attention_no_mfma;   // 1 = grouped-query decode attention stays on the float32 vector kernel
   int int8_gemm_tile;      // 0 = heuristic, else 128 or 256 rows per workgroup in the many-row int8 matmul
 };
 Options &options();

@@ -168,3 +168,39 @@ def test_fused_prefill_matches_stock_prefill(fully_causal):
             model_mod.FUSED_DECODE = True
     err = (out[True] - out[False]).abs().max() / out[False].abs().max()
     assert err < 2e-2, err
+
+
+@pytest.mark.parametrize("n_head,n_kv", [(16, 4), (64, 8), (32, 2), (12, 2)])
+@pytest.mark.parametrize("s_max,pos", [(96, 0), (96, 31), (96, 32), (96, 41), (640, 575), (300, 299)])
+def test_grouped_query_attention_on_matrix_cores_matches_sdpa_and_vector_kernel(n_head, n_kv, s_max, pos):
+    """4 .. 16 query heads per kv head at head_dim 128 take the MFMA kernel (both cache lengths: 4 and 8 waves): against
+    stock SDPA on the same cache, with and without left padding, and against the float32 vector kernel (the two differ
+    by the bfloat16 rounding of the softmax weights only)."""
+    from easy_to_hard_amd import _lib
+
+    d, bsz = 128, 3
+    rep = n_head // n_kv
+    gen = torch.Generator().manual_seed(n_head * 7 + pos)
+    q = torch.randn((bsz, n_head, d), generator=gen).to(torch.bfloat16).to(DEV)
+    kc = torch.randn((bsz, n_kv, s_max, d), generator=gen).to(torch.bfloat16).to(DEV)
+    vc = torch.randn((bsz, n_kv, s_max, d), generator=gen).to(torch.bfloat16).to(DEV)
+    input_pos = torch.tensor([pos], device=DEV)
+    for left_pad in (None, torch.tensor([0, min(7, pos), pos], device=DEV)):
+        mask = (torch.arange(s_max, device=DEV) <= pos)[None, None, None, :]
+        if left_pad is not None:
+            vis = torch.arange(s_max, device=DEV).view(1, -1) >= left_pad.view(-1, 1)
+            mask = torch.logical_and(mask, vis[:, None, None, :])
+            mask = torch.logical_or(mask, (torch.arange(s_max, device=DEV) == pos)[None, None, None, :])
+        kk = kc.repeat_interleave(rep, dim=1).float()
+        vv = vc.repeat_interleave(rep, dim=1).float()
+        ref = F.scaled_dot_product_attention(q.float()[:, :, None, :], kk, vv, attn_mask=mask).squeeze(2)
+        y = ops.decode_attention(q, kc, vc, input_pos, left_pad)
+        scale = float(ref.abs().max())
+        assert (y.float() - ref).abs().max() < 1e-2 * scale
+        if rep in (4, 8):  # the vector kernel is instantiated for 1, 2, 4 and 8 heads per kv head
+            _lib.set_option("attention_no_mfma", 1)
+            try:
+                y_vec = ops.decode_attention(q, kc, vc, input_pos, left_pad)
+            finally:
+                _lib.set_option("attention_no_mfma", 0)
+            assert (y.float() - y_vec.float()).abs().max() < 1e-2 * scale
