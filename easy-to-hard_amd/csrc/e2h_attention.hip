@@ -543,8 +543,9 @@ int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const
                      const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
   const int nw = options().attention_waves ? options().attention_waves : (S > 256 ? 8 : 4);
   if (D == 128 && rep >= 4 && rep <= 16 && !options().attention_no_mfma) {
-    // several query heads per K / V row: both products on the matrix cores
-    if (nw == 8)
+    // several query heads per K / V row: both products on the matrix cores; four waves measured faster than eight
+    // (three workgroups fit a CU instead of one)
+    if (options().attention_waves == 8)
       hipLaunchKernelGGL(decode_attention_gqa_kernel<8>, grid, dim3(512), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale);
     else
       hipLaunchKernelGGL(decode_attention_gqa_kernel<4>, grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale);
