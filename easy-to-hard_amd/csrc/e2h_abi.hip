@@ -87,6 +87,16 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.attention_waves = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "int8_gemm_waves")) {
+    if (value != 0 && value != 4 && value != 8) return E2H_ERR_BAD_OPTION;
+    o.int8_gemm_waves = value;
+    return E2H_OK;
+  }
+  if (!strcmp(name, "int8_gemm_wave_cols")) {
+    if (value != 0 && value != 2 && value != 4) return E2H_ERR_BAD_OPTION;
+    o.int8_gemm_wave_cols = value;
+    return E2H_OK;
+  }
   if (!strcmp(name, "int8_gemm_tile")) {
     if (value != 0 && value != 128 && value != 256) return E2H_ERR_BAD_OPTION;
     o.int8_gemm_tile = value;

@@ -50,6 +50,8 @@ struct Options {
   int attention_waves;     // 0 = by cache length, else 4 or 8 waves per decode-attention workgroup
   int attention_no_mfma;   // 1 = grouped-query decode attention stays on the float32 vector kernel
   int int8_gemm_tile;      // 0 = heuristic, else 128 or 256 rows per workgroup in the many-row int8 matmul
+  int int8_gemm_waves;     // 4 = the 256-row workgroup runs as four waves of 128 x 128 outputs each
+  int int8_gemm_wave_cols; // with four waves: 4 = every wave 256 rows x 64 columns instead
 };
 Options &options();
 
@@ -65,9 +67,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, ui
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 #endif
 
-// many-row int8 matmul on 32x32 MFMA tiles (e2h_int8_gemm.hip); xsum: scratch for the sums of x, xsum_bytes large
-int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, float *xsum, int64_t xsum_bytes, int M,
-                int N, int K, hipStream_t stream);
+// many-row int8 matmul on 32x32 MFMA tiles (e2h_int8_gemm.hip); needs no scratch memory
+int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int M, int N, int K, hipStream_t stream);
 
 // streaming int8 matmul (e2h_int8_stream.hip)
 int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int M, int N, int K, void *workspace,

@@ -27,6 +27,64 @@ __device__ __forceinline__ bf16x8_t unpack_word(uint32_t w, const UnpackConsts &
   return __builtin_bit_cast(bf16x8_t, u);
 }
 
+// ---- output of the 32x32-tile kernels ----------------------------------------------------------------------------
+// A wave holds RT x CT accumulator tiles of v_mfma_f32_32x32x*: lane (h, n) = column n of a tile, element e = row
+// 8 (e / 4) + 4 h + e % 4.  Stored straight from that layout every lane writes 2 bytes per instruction; instead each
+// 32-row slab goes through a wave-private LDS tile (32 rows x 32 CT columns, row stride kTileStride bytes) and leaves
+// as 16-byte pieces of output rows.  Rounding uses the packed hardware convert (round to nearest even, two values per
+// instruction).  kScale: the int8 contract y = bf16(bf16(acc) * scale[column]); otherwise y = bf16(acc).
+// Needs N % 8 == 0 and a 16-byte aligned y (the caller checks and otherwise stores element-wise).
+typedef float e2h_float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 e2h_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float e2h_f32x16_t __attribute__((ext_vector_type(16)));
+
+template <int CT>
+struct TileStore {
+  static constexpr int kTileStride = 64 * CT + 16;
+  static constexpr int kBytesPerWave = 32 * kTileStride;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16x2_rne(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(e2h_float2_t{a, b}, e2h_bf16x2_t));
+}
+
+template <int RT, int CT, bool kScale>
+__device__ __forceinline__ void store_tiles_via_lds(const e2h_f32x16_t (&acc)[CT][RT], const float (&scale)[CT], uint8_t *tile,
+                                                    uint16_t *__restrict__ y, int row0, int col0, int M, int N, int lane) {
+  constexpr int kTileStride = TileStore<CT>::kTileStride;
+  constexpr int kPiecesPerRow = 4 * CT;             // 16-byte pieces per tile row
+  constexpr int kRowsPerPass = 64 / kPiecesPerRow;  // tile rows one 64-lane read covers
+  const int n = lane & 31, h = lane >> 5;
+  const bool odd = n & 1;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        // own = (row e, row e + 1) of column n
+        uint32_t own = pack_bf16x2_rne(acc[ct][rt][e], acc[ct][rt][e + 1]);
+        if (kScale) {
+          const float t0 = __builtin_bit_cast(float, own << 16), t1 = __builtin_bit_cast(float, own & 0xFFFF0000u);
+          own = pack_bf16x2_rne(t0 * scale[ct], t1 * scale[ct]);
+        }
+        // neighbouring lanes (columns n, n ^ 1) trade words: even lanes keep row e of both columns (the low halves),
+        // odd lanes row e + 1 (the high halves)
+        const uint32_t nbr = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(own), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+        const uint32_t word = __builtin_amdgcn_perm(nbr, own, odd ? 0x03020706u : 0x05040100u);
+        const int row = 8 * (e >> 2) + 4 * h + (e & 3) + (odd ? 1 : 0);
+        *reinterpret_cast<uint32_t *>(tile + row * kTileStride + (32 * ct + (n & ~1)) * 2) = word;
+      }
+#pragma unroll
+    for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
+      const int trow = pass * kRowsPerPass + lane / kPiecesPerRow, piece = lane % kPiecesPerRow;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t *>(tile + trow * kTileStride + piece * 16);
+      const int row = row0 + 32 * rt + trow, col = col0 + 8 * piece;
+      if (row < M && col < N) *reinterpret_cast<u32x4_t *>(y + static_cast<size_t>(row) * N + col) = v;
+    }
+  }
+}
+
 // One pass over x: sums over every (row, quantization group), float32, stored group-major [K/G][stride]
 // (defined in e2h_int4_mm.hip; groupsize in {32, 64, 128}).
 int launch_x_group_sums(const uint16_t *x, float *out, int M, int K, int stride, int groupsize, hipStream_t stream);

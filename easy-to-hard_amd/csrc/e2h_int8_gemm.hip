@@ -3,11 +3,8 @@
 // Same contract as e2h_int8_mm (WeightOnlyInt8Linear.forward, reference models/quantize.py:428-429):
 //   y = bf16( bf16( x @ q^T ) * scales ),   q int8 [N][K] row-major, K % 128 == 0, 16-byte aligned rows.
 //
-// int8 -> bfloat16 without sign handling: u = q + 128 (one XOR per four codes) lies in [0, 255] and is exactly
-// representable in bfloat16's 8 significant bits, so each code costs one byte-to-float convert and half a byte
-// permute.  The offset is taken back out through the accumulators' initial value
-//   acc0[m,n] = -128 * sum_k x[m,k],
-// built before the main loop from per-128 sums of x (a one-pass pre-kernel) with v_mfma_f32_32x32x2_f32.
+// int8 -> bfloat16: a sign-extending byte-to-float convert per code (the value has at most 8 significant bits, so
+// the high half of the float is the exact bfloat16) and half a byte permute to pack two of them.
 //
 // Main loop, v_mfma_f32_32x32x16_bf16: lane L = 32*h + n supplies weight row n0 + n; per 32-wide k span t its B
 // operands are the 16 bytes k = 32 t + 16 h .. +15, bytes 0..7 feeding step (t, 0) and bytes 8..15 step (t, 1).  The
@@ -28,26 +25,23 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kFragB8 = 1024 + 32;
 
-// four codes (one dword, already offset to unsigned) -> two dwords of bfloat16 pairs
+// four codes (one dword) -> two dwords of bfloat16 pairs
 __device__ __forceinline__ void bytes4_to_bf16(uint32_t t, uint32_t &lo, uint32_t &hi) {
-  const float f0 = static_cast<float>(t & 0xFFu), f1 = static_cast<float>((t >> 8) & 0xFFu);
-  const float f2 = static_cast<float>((t >> 16) & 0xFFu), f3 = static_cast<float>(t >> 24);
+  const float f0 = static_cast<float>(static_cast<int8_t>(t & 0xFFu)), f1 = static_cast<float>(static_cast<int8_t>((t >> 8) & 0xFFu));
+  const float f2 = static_cast<float>(static_cast<int8_t>((t >> 16) & 0xFFu)), f3 = static_cast<float>(static_cast<int8_t>(t >> 24));
   // high halves of two floats (exact: the values have at most 8 significant bits)
   lo = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0), 0x07060302u);
   hi = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
 }
 
 // WR x WC waves per workgroup, RT x CT tiles of 32 x 32 outputs per wave, CK = k per staged chunk (64 or 128).
-// <2, 4, 2, 2, 128>: 8 waves, 128 x 256 outputs per workgroup.  <2, 4, 4, 2, 64>: 8 waves, 256 x 256 outputs per
-// workgroup, every wave 128 rows x 64 columns (128 accumulator registers): a converted weight fragment feeds four row
-// tiles instead of two, so conversions and LDS reads per MFMA drop by 40 %; the k chunk halves to keep both stages
-// within the LDS.  (Four waves with 4 x 4 tiles and the accumulators in the accumulation registers measured slower:
-// one wave per SIMD leaves nothing to cover its LDS and conversion latencies.)
+// <2, 4, 2, 2, 128>: 8 waves, 128 x 256 outputs per workgroup, the form for row counts that leave CUs idle with
+// 256-row workgroups.  <2, 4, 4, 2, 64>: 8 waves, 256 x 256 outputs per workgroup, every wave 128 rows x 64 columns
+// (128 accumulator registers); kept selectable as the comparison for int8_gemm128_kernel below, which replaced it.
 template <int WR, int WC, int RT, int CT, int CK>
 __global__ __launch_bounds__(64 * WR * WC) void int8_gemm32_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
-                                                                   const uint16_t *__restrict__ scales, uint16_t *__restrict__ y,
-                                                                   const float *__restrict__ xsum, int xsum_stride, int M, int N, int K,
-                                                                   int n_col_blocks, int cbx) {
+                                                                   const uint16_t *__restrict__ scales, uint16_t *__restrict__ y, int M, int N,
+                                                                   int K, int n_col_blocks, int cbx) {
   constexpr int kThreads = 64 * WR * WC;
   constexpr int kRows = 32 * RT * WR, kCols = 32 * CT * WC;
   constexpr int SPC = CK / 16;                        // MFMA steps per chunk = activation fragments per 32-row tile
@@ -77,38 +71,17 @@ __global__ __launch_bounds__(64 * WR * WC) void int8_gemm32_kernel(const uint16_
   const int row0 = rb * kRows + wr * (32 * RT);
   const int col0 = cb * kCols + wc * (32 * CT);
   const int nchunks = K / CK;
-  const int nsums = K / 128;  // the pre-pass leaves sums of x over spans of 128
 
   const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(q, static_cast<uint32_t>(static_cast<size_t>(N) * K));
   const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
-  const __amdgpu_buffer_rsrc_t xs_rsrc = make_rsrc(xsum, static_cast<uint32_t>(static_cast<size_t>(nsums) * xsum_stride * 4));
 
-  // ---- accumulators start at -128 * sum_k x[m,k] (float32 MFMAs over the per-chunk sums of x) ------------------
-  // (the value does not depend on the column: one MFMA chain per row tile, copied to the tile's columns)
   f32x16_t acc[CT][RT];
-  {
-    f32x16_t init[RT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) init[rt][e] = 0.f;
-    uint32_t xslane[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) xslane[rt] = static_cast<uint32_t>(h * xsum_stride + row0 + 32 * rt + n) * 4u;
-#pragma unroll 4
-    for (int g0 = 0; g0 < nsums; g0 += 2) {  // lanes with h = 1 take span g0 + 1 (reads past the last one return 0)
-      float a[RT];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-        a[rt] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xs_rsrc, xslane[rt], static_cast<uint32_t>(g0) * xsum_stride * 4u, 0));
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) init[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rt], -128.0f, init[rt], 0, 0, 0);
-    }
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) acc[ct][rt] = init[rt];
-  }
+      for (int e = 0; e < 16; ++e) acc[ct][rt][e] = 0.f;
 
   // ---- staging.  Activations: piece (row, w), k = 8 w .. 8 w + 7 = 32 t + 16 h + 8 a with w = 4 t + 2 h + a, goes to
   // fragment (row tile, step 2 t + a), lane (h, row % 32).  Weights: piece (col, pc), bytes 16 pc .. 16 pc + 15 =
@@ -168,8 +141,8 @@ __global__ __launch_bounds__(64 * WR * WC) void int8_gemm32_kernel(const uint16_
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
           uint32_t u0, u1, u2, u3;
-          bytes4_to_bf16(wq[ct][2 * a] ^ 0x80808080u, u0, u1);
-          bytes4_to_bf16(wq[ct][2 * a + 1] ^ 0x80808080u, u2, u3);
+          bytes4_to_bf16(wq[ct][2 * a], u0, u1);
+          bytes4_to_bf16(wq[ct][2 * a + 1], u2, u3);
           const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, u32x4_t{u0, u1, u2, u3});
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) acc[ct][rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[rt], wf, acc[ct][rt], 0, 0, 0);
@@ -191,29 +164,243 @@ __global__ __launch_bounds__(64 * WR * WC) void int8_gemm32_kernel(const uint16_
   }
 
   // ---- store with the reference's two roundings: bf16(acc), then bf16(t * scale) ----------------------------------
+  float scale[CT];
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     const int col = col0 + 32 * ct + n;
-    const float scale = bf16_to_f32(scales[col < N ? col : N - 1]);
+    scale[ct] = bf16_to_f32(scales[col < N ? col : N - 1]);
+  }
+  if ((N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+    // (the barrier that ended the last chunk left every wave done with the stages)
+    store_tiles_via_lds<RT, CT, true>(acc, scale, lds + wave * TileStore<CT>::kBytesPerWave, y, row0, col0, M, N, lane);
+    return;
+  }
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = col0 + 32 * ct + n;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int row = row0 + 32 * rt + 8 * (e >> 2) + 4 * h + (e & 3);
-        if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = f32_to_bf16_rne(bf16_round(acc[ct][rt][e]) * scale);
+        if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = f32_to_bf16_rne(bf16_round(acc[ct][rt][e]) * scale[ct]);
+      }
+  }
+}
+
+
+// Four waves, 256 x 256 outputs per workgroup: <2, 2> every wave 128 rows x 128 columns, <1, 4> 256 rows x 64
+// columns (the default: a converted weight fragment then feeds eight MFMAs and no two waves convert the same one).
+// 256 accumulator registers per lane: one wave per SIMD owns the whole 512-register budget, each fragment read from
+// LDS feeds more MFMAs, and the LDS carries about half the bytes per MFMA of the eight-wave forms.  With nothing else
+// on the SIMD to cover latencies the wave pipelines itself (see the slot schedule in the body).  Codes are converted
+// with sign-extending byte-to-float instructions, so there is no +128 offset to take back out: no pass over x
+// beforehand, no accumulator prologue.  Measured against the eight-wave 256-row form on the same GPU, 7B shapes at
+// 8192 rows: 4 % (12288 x 4096) to 14 % (4096 x 11008) less time.  What bounds it: with every matrix pipeline busy
+// the chip clocks near 1.6 GHz (the same loop with the MFMAs alone reaches 1650 TFLOP/s, which the bfloat16 library
+// matmul nearly attains); LDS reads, staging stores and loads each add 8 - 14 % on top when timed by omission.
+template <int WR, int WC, int CK>
+__global__ __launch_bounds__(256) void int8_gemm128_kernel(const uint16_t *__restrict__ x, const int8_t *__restrict__ q,
+                                                           const uint16_t *__restrict__ scales, uint16_t *__restrict__ y, int M, int N, int K,
+                                                           int n_col_blocks, int cbx) {
+  static_assert(WR * WC == 4, "four waves");
+  constexpr int RT = 8 / WR, CT = 8 / WC;  // 256 x 256 outputs per workgroup
+  constexpr int kThreads = 256;
+  constexpr int kRows = 256, kCols = 256;
+  constexpr int SPC = CK / 16, TPC = CK / 32;
+  constexpr int kStageX = (RT * WR) * SPC * kFragB8;
+  constexpr int kStageW = (CT * WC) * TPC * kFragB8;
+  constexpr int PX = CK / 8, PW = CK / 16;
+  constexpr int kXRowsPerPass = kThreads / PX;
+  constexpr int kXPieces = kRows / kXRowsPerPass;
+  constexpr int kWColsPerPass = kThreads / PW;
+  constexpr int kWPieces = kCols / kWColsPerPass;
+  static_assert(kXRowsPerPass % 32 == 0 && kWColsPerPass % 32 == 0, "staging passes cover whole 32-wide tiles");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * (kStageX + kStageW)];
+  uint8_t *const lds_w = lds + 2 * kStageX;
+
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int cb = xcd + 8 * (slot % cbx);
+  const int rb = slot / cbx;
+  if (cb >= n_col_blocks) return;  // grid padding; uniform, before any barrier
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = wave / WC, wc = wave % WC;
+  const int n = lane & 31, h = lane >> 5;
+  const int row0 = rb * kRows + wr * (32 * RT);
+  const int col0 = cb * kCols + wc * (32 * CT);
+  const int nchunks = K / CK;
+
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(q, static_cast<uint32_t>(static_cast<size_t>(N) * K));
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x, static_cast<uint32_t>(static_cast<size_t>(M) * K * 2));
+
+  f32x16_t acc[CT][RT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[ct][rt][e] = 0.f;
+
+  // staging: the same piece -> fragment maps as in int8_gemm32_kernel
+  const int xr0 = tid / PX, xw = tid % PX;
+  uint32_t xsrc[kXPieces];
+#pragma unroll
+  for (int i = 0; i < kXPieces; ++i) {
+    int row = rb * kRows + xr0 + kXRowsPerPass * i;
+    row = row < M ? row : M - 1;
+    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + xw * 8) * 2);
+  }
+  const int xdst0 = ((xr0 >> 5) * SPC + 2 * (xw >> 2) + (xw & 1)) * kFragB8 + (((xw >> 1) & 1) * 32 + (xr0 & 31)) * 16;
+  const int wc0 = tid / PW, wpc = tid % PW;
+  uint32_t wsrc[kWPieces];
+#pragma unroll
+  for (int i = 0; i < kWPieces; ++i) {
+    int col = cb * kCols + wc0 + kWColsPerPass * i;
+    col = col < N ? col : N - 1;
+    wsrc[i] = static_cast<uint32_t>(static_cast<size_t>(col) * K + wpc * 16);
+  }
+  const int wdst0 = ((wc0 >> 5) * TPC + (wpc >> 1)) * kFragB8 + ((wpc & 1) * 32 + (wc0 & 31)) * 16;
+
+  static_assert(kXPieces + kWPieces == 12 && SPC == 4, "the slot schedule below is written for 64-wide chunks");
+  struct Staged {
+    u32x4_t p[kXPieces + kWPieces];  // activation pieces, then weight pieces
+  };
+  auto load_piece = [&](Staged &r, int ci, int i) {
+    const int cc = ci < nchunks ? ci : nchunks - 1;
+    if (i < kXPieces)
+      r.p[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(cc) * (CK * 2), 0);
+    else
+      r.p[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, wsrc[i - kXPieces], static_cast<uint32_t>(cc) * CK, 0);
+  };
+  auto store_piece = [&](const Staged &r, int parity, int i) {
+    if (i < kXPieces)
+      *reinterpret_cast<u32x4_t *>(lds + (parity & 1) * kStageX + xdst0 + i * (kXRowsPerPass / 32) * (SPC * kFragB8)) = r.p[i];
+    else
+      *reinterpret_cast<u32x4_t *>(lds_w + (parity & 1) * kStageW + wdst0 + (i - kXPieces) * (kWColsPerPass / 32) * (TPC * kFragB8)) = r.p[i];
+  };
+
+  const int x_frag0 = (wr * RT) * (SPC * kFragB8) + lane * 16;
+  const int w_frag0 = (wc * CT) * (TPC * kFragB8) + lane * 16;
+  bf16x8_t af[2][RT];
+  u32x4_t wq[2][CT];
+  auto read_a = [&](int parity, int s, int rt) {
+    return *reinterpret_cast<const bf16x8_t *>(lds + (parity & 1) * kStageX + x_frag0 + (rt * SPC + s) * kFragB8);
+  };
+  auto read_w = [&](int parity, int t, int ct) {
+    return *reinterpret_cast<const u32x4_t *>(lds_w + (parity & 1) * kStageW + w_frag0 + (ct * TPC + t) * kFragB8);
+  };
+
+  // One MFMA occupies the matrix pipeline for 32 cycles and the wave issues in order, with no second wave on its SIMD
+  // to fill gaps.  So everything else is cut into pieces that fit behind one MFMA each and fenced there: the
+  // conversion of the next weight fragment (14 vector instructions in four parts), and one memory instruction per
+  // slot -- a fragment read for the next step, a staging store of the next chunk, or a load two chunks ahead.
+  uint32_t cv[4];  // the fragment being converted
+  auto convert_part = [&](uint32_t d0, uint32_t d1, int part) {
+    // sign-extending byte-to-float converts (one instruction per code), high halves of two floats per permute: exact,
+    // |q| <= 128 has at most 8 significant bits
+    const uint32_t t = part < 2 ? d0 : d1;
+    if ((part & 1) == 0) {
+      const float f0 = static_cast<float>(static_cast<int8_t>(t & 0xFFu)), f1 = static_cast<float>(static_cast<int8_t>((t >> 8) & 0xFFu));
+      cv[part] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f1), __builtin_bit_cast(uint32_t, f0), 0x07060302u);
+    } else {
+      const float f2 = static_cast<float>(static_cast<int8_t>((t >> 16) & 0xFFu)), f3 = static_cast<float>(static_cast<int8_t>(t >> 24));
+      cv[part] = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, f3), __builtin_bit_cast(uint32_t, f2), 0x07060302u);
+    }
+  };
+  bf16x8_t wf;  // converted fragment of the column tile whose MFMAs come next
+
+  // Slot j = 0 .. 15 of step s of chunk ci, whose register set r holds chunk ci + 1 (loaded two chunks ago: the
+  // memory round trip under load is longer than one chunk):
+  //   j < RT: activation fragment j of the next step           j < CT, s odd: weight codes of the next 32-wide span
+  //   j = 8 .. 11, s < 3: staging store of piece 4 s + j - 8     j = 12 .. 15, s < 3: load of that piece of chunk ci + 3
+  // The last step's reads address the next chunk's stage, behind the chunk's only barrier.
+  auto slot_op = [&](int ci, Staged &r, int s, int j) {
+    const int t = s >> 1;
+    const bool last = s + 1 == SPC;
+    if (j < RT) af[(s + 1) & 1][j] = last ? read_a(ci + 1, 0, j) : read_a(ci, s + 1, j);
+    if (j < CT && (s & 1)) wq[(t + 1) & 1][j] = last ? read_w(ci + 1, 0, j) : read_w(ci, t + 1, j);
+    if (!last && j >= 8 && j < 12) store_piece(r, ci + 1, 4 * s + j - 8);
+    if (!last && j >= 12) load_piece(r, ci + 3, 4 * s + j - 12);
+  };
+  auto chunk = [&](int ci, Staged &r) {
+#pragma unroll
+    for (int s = 0; s < SPC; ++s) {
+      const int t = s >> 1, a = s & 1;
+      if (s + 1 == SPC) lds_barrier();  // staging stores of this chunk visible, every wave done reading this stage
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        // the fragment to convert meanwhile: the next column tile's, or the first one of the following step
+        const u32x4_t &nx = ct + 1 < CT ? wq[t & 1][ct + 1] : (a ? wq[(t + 1) & 1][0] : wq[t & 1][0]);
+        const int na = ct + 1 < CT ? a : (a ^ 1);
+        const uint32_t d0 = nx[2 * na], d1 = nx[2 * na + 1];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          acc[ct][rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[s & 1][rt], wf, acc[ct][rt], 0, 0, 0);
+          constexpr int kEvery = RT / 4;  // conversion parts per column tile: 4, spread over its RT MFMAs
+          if (rt % kEvery == kEvery - 1) convert_part(d0, d1, rt / kEvery);
+          slot_op(ci, r, s, ct * RT + rt);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        wf = __builtin_bit_cast(bf16x8_t, u32x4_t{cv[0], cv[1], cv[2], cv[3]});
+      }
+    }
+  };
+
+  Staged st[2];
+#pragma unroll
+  for (int i = 0; i < 12; ++i) load_piece(st[0], 0, i);
+#pragma unroll
+  for (int i = 0; i < 12; ++i) store_piece(st[0], 0, i);
+#pragma unroll
+  for (int i = 0; i < 12; ++i) load_piece(st[1], 1, i);
+#pragma unroll
+  for (int i = 0; i < 12; ++i) load_piece(st[0], 2, i);
+  lds_barrier();
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) af[0][rt] = read_a(0, 0, rt);
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) wq[0][ct] = read_w(0, 0, ct);
+#pragma unroll
+  for (int part = 0; part < 4; ++part) convert_part(wq[0][0][0], wq[0][0][1], part);
+  wf = __builtin_bit_cast(bf16x8_t, u32x4_t{cv[0], cv[1], cv[2], cv[3]});
+  for (int ci = 0; ci < nchunks; ci += 2) {  // K % 128 == 0: an even number of 64-wide chunks
+    chunk(ci, st[1]);
+    chunk(ci + 1, st[0]);
+  }
+
+  // ---- store with the reference's two roundings: bf16(acc), then bf16(t * scale) ----------------------------------
+  float scale[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = col0 + 32 * ct + n;
+    scale[ct] = bf16_to_f32(scales[col < N ? col : N - 1]);
+  }
+  if ((N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+    lds_barrier();  // the staging stages are dead from here on
+    store_tiles_via_lds<RT, CT, true>(acc, scale, lds + wave * TileStore<CT>::kBytesPerWave, y, row0, col0, M, N, lane);
+    return;
+  }
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int col = col0 + 32 * ct + n;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = row0 + 32 * rt + 8 * (e >> 2) + 4 * h + (e & 3);
+        if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = f32_to_bf16_rne(bf16_round(acc[ct][rt][e]) * scale[ct]);
       }
   }
 }
 
 }  // namespace
 
-int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, float *xsum, int64_t xsum_bytes, int M,
-                int N, int K, hipStream_t stream) {
+int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint16_t *y, int M, int N, int K, hipStream_t stream) {
   if (K % 128 != 0) return E2H_ERR_BAD_SHAPE;
-  const int stride = ((M + 63) / 64) * 64;
-  if (static_cast<int64_t>(K / 128) * stride * 4 > xsum_bytes) return E2H_ERR_BAD_SHAPE;
-  const int rc = launch_x_group_sums(x, xsum, M, K, stride, 128, stream);
-  if (rc != E2H_OK) return rc;
   // 256 x 256 or 128 x 256 outputs per workgroup (one workgroup per CU either way).  A 256-row workgroup takes
   // about 1.8 x as long as a 128-row one (measured: 10 % more throughput), so it wins exactly when it needs fewer than
   // 1 / 1.8 as many rounds of workgroups over the chip's 256 CUs.
@@ -226,12 +413,21 @@ int int8_gemm32(const uint16_t *x, const int8_t *q, const uint16_t *scales, uint
   const int cbx = (n_col_blocks + 7) / 8;
   const long long wgs = 8LL * cbx * n_row_blocks;
   if (wgs > 0x7FFFFFFFLL) return E2H_ERR_BAD_SHAPE;
+  if (big && options().int8_gemm_waves != 8) {
+    if (options().int8_gemm_wave_cols == 2)
+      hipLaunchKernelGGL((int8_gemm128_kernel<2, 2, 64>), dim3(static_cast<unsigned>(wgs)), dim3(256), 0, stream, x, q, scales, y, M, N, K,
+                         n_col_blocks, cbx);
+    else
+      hipLaunchKernelGGL((int8_gemm128_kernel<1, 4, 64>), dim3(static_cast<unsigned>(wgs)), dim3(256), 0, stream, x, q, scales, y, M, N, K,
+                         n_col_blocks, cbx);
+    return launch_status();
+  }
   if (big)
-    hipLaunchKernelGGL((int8_gemm32_kernel<2, 4, 4, 2, 64>), dim3(static_cast<unsigned>(wgs)), dim3(512), 0, stream, x, q, scales, y, xsum,
-                       stride, M, N, K, n_col_blocks, cbx);
+    hipLaunchKernelGGL((int8_gemm32_kernel<2, 4, 4, 2, 64>), dim3(static_cast<unsigned>(wgs)), dim3(512), 0, stream, x, q, scales, y, M, N, K,
+                       n_col_blocks, cbx);
   else
-    hipLaunchKernelGGL((int8_gemm32_kernel<2, 4, 2, 2, 128>), dim3(static_cast<unsigned>(wgs)), dim3(512), 0, stream, x, q, scales, y, xsum,
-                       stride, M, N, K, n_col_blocks, cbx);
+    hipLaunchKernelGGL((int8_gemm32_kernel<2, 4, 2, 2, 128>), dim3(static_cast<unsigned>(wgs)), dim3(512), 0, stream, x, q, scales, y, M, N, K,
+                       n_col_blocks, cbx);
   return launch_status();
 }
 

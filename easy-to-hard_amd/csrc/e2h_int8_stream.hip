@@ -444,15 +444,10 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
     int rc;
     const long long wgs32 = static_cast<long long>((a.M + 127) / 128) * ((N + 127) / 128);
     const bool use32 = options().int4_gemm32_min_rows > 0 ? a.M >= options().int4_gemm32_min_rows : wgs32 >= 320;
-    if (mt == 4 && use32 && !options().int4_no_gemm32 && workspace && static_cast<int64_t>(N) * K < (int64_t{1} << 32)) {
-      // many rows: 32x32-tile kernel; the sums of x go to the partial-tile area of the workspace (no K split here)
-      const int64_t avail = workspace_bytes - static_cast<int64_t>(kTicketBytes8);
-      const int64_t need = static_cast<int64_t>(K / 128) * (((a.M + 63) / 64) * 64) * 4;
-      if (need <= avail) {
-        rc = int8_gemm32(a.x, q, scales, a.y, reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + kTicketBytes8), avail, a.M, N, K, stream);
-        if (rc != E2H_OK) return rc;
-        continue;
-      }
+    if (mt == 4 && use32 && !options().int4_no_gemm32 && static_cast<int64_t>(N) * K < (int64_t{1} << 32)) {
+      rc = int8_gemm32(a.x, q, scales, a.y, a.M, N, K, stream);  // many rows: 32x32-tile kernels, no K split, no scratch
+      if (rc != E2H_OK) return rc;
+      continue;
     }
     if (mt == 1) rc = t == 2 ? (wk == 2 ? launch8<1, 2, 4, 2>(a) : launch8<1, 2, 4, 1>(a)) : (wk == 2 ? launch8<1, 1, 4, 2>(a) : launch8<1, 1, 4, 1>(a));
     else if (mt == 2) rc = t == 2 ? (wk == 2 ? launch8<2, 2, 4, 2>(a) : launch8<2, 2, 4, 1>(a)) : (wk == 2 ? launch8<2, 1, 4, 2>(a) : launch8<2, 1, 4, 1>(a));

@@ -398,10 +398,10 @@ def test_int4_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, g):
     assert (yi.float() - yi2.float()).abs().max().item() <= 2.0 ** -7 * yi2.float().abs().max().item()
 
 
-@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("tile,waves,wave_cols", [(128, 0, 0), (256, 8, 0), (256, 4, 2), (256, 4, 4)])
 @pytest.mark.parametrize("m,n,k", [(65, 1, 128), (130, 272, 1024), (257, 136, 384), (512, 4096, 4096), (300, 2, 4096), (700, 520, 640)])
-def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile):
-    """The 32x32-tile int8 kernels (many rows; 128 x 256 and 256 x 256 outputs per workgroup) against the oracle, the
+def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile, waves, wave_cols):
+    """The 32x32-tile int8 kernels (many rows; 128 x 256 and 256 x 256 outputs per workgroup, the latter with eight or four waves) against the oracle, the
     reference's two-rounding form and the 16x16-tile kernel: ragged M and N (incl. the 2-row reward head), a single
     chunk, odd chunk counts, and rows with extreme codes (-128 / 127) so that the +128 offset and its correction are
     exercised at both ends."""
@@ -413,6 +413,8 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile):
     x = randn_bf16((m, k), std=1.0, seed=m + 2)
     _lib.set_option("int4_gemm32_min_rows", 65)
     _lib.set_option("int8_gemm_tile", tile)
+    _lib.set_option("int8_gemm_waves", waves)
+    _lib.set_option("int8_gemm_wave_cols", wave_cols)
     try:
         y, _ = _check_int8(x, q, s, q_d, s_d)
         xi = torch.randint(-1, 2, (m, k), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
@@ -420,6 +422,8 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile):
     finally:
         _lib.set_option("int4_gemm32_min_rows", 0)
         _lib.set_option("int8_gemm_tile", 0)
+        _lib.set_option("int8_gemm_waves", 0)
+        _lib.set_option("int8_gemm_wave_cols", 0)
     _lib.set_option("int4_no_gemm32", 1)
     try:
         y2, _ = _check_int8(x, q, s, q_d, s_d)
