@@ -1,6 +1,8 @@
 """GPU parity of the dequant GEMV / skinny GEMM kernels against the float32 dequantize-then-matmul
 oracle, through the C ABI.  Gate: max|y - y_ref| / max|y_ref| <= 1e-2 (bf16 outputs)."""
 
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -435,6 +437,41 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile, waves, w
     assert torch.equal(yi, yi2)
     y_rr = qo.int8_linear_reference_rounding(bf16_to_np(xi), q, s)
     assert np.array_equal(bf16_to_np(yi), y_rr)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["int8", "int4"])
+def test_many_row_kernels_with_an_output_that_is_only_2_byte_aligned(mode):
+    """The 32x32-tile kernels write 16-byte pieces of output rows; the C ABI only promises a 2-byte aligned y, so an
+    output that starts 2 bytes into an allocation must take the element-wise stores and give the very same values."""
+    m, n, k, g = 300, 264, 512, 128
+    x = randn_bf16((m, k), std=1.0, seed=5).to(DEV)
+    buf = torch.zeros(m * n + 8, dtype=torch.bfloat16, device=DEV)
+    ws = ops._workspace(x.device)
+    lib = ops._lib_for(x)
+    _lib.set_option("int4_gemm32_min_rows", 65)
+    try:
+        if mode == "int8":
+            q, s, q_d, s_d = _int8_case(n, k, seed=11)
+            y_ref = ops.int8_mm_direct(x, q_d, s_d)
+            for tile in (128, 256):
+                _lib.set_option("int8_gemm_tile", tile)
+                buf.zero_()
+                rc = lib.e2h_int8_mm(ops._ptr(x), ops._ptr(q_d), ops._ptr(s_d), ctypes.c_void_p(buf.data_ptr() + 2), m, n, k, ops._ptr(ws), ws.numel(), ops._stream(x))
+                _lib.check(rc, "e2h_int8_mm")
+                assert torch.equal(buf[1:1 + m * n].view(m, n), y_ref)
+                assert buf[0].item() == 0 and buf[1 + m * n:].abs().max().item() == 0
+        else:
+            codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=12)
+            y_ref = ops.int4_mm_direct(x, packed_d, g, sz_d)
+            rc = lib.e2h_int4_mm(ops._ptr(x), ops._ptr(packed_d), ops._ptr(sz_d), ctypes.c_void_p(buf.data_ptr() + 2), m, n, k, g, 8, ops._ptr(ws), ws.numel(),
+                                 ops._stream(x))
+            _lib.check(rc, "e2h_int4_mm")
+            assert torch.equal(buf[1:1 + m * n].view(m, n), y_ref)
+            assert buf[0].item() == 0 and buf[1 + m * n:].abs().max().item() == 0
+    finally:
+        _lib.set_option("int4_gemm32_min_rows", 0)
+        _lib.set_option("int8_gemm_tile", 0)
 
 
 @pytest.mark.gpu
