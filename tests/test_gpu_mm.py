@@ -440,6 +440,31 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile, waves, w
 
 
 @pytest.mark.gpu
+def test_int8_many_rows_at_the_reward_scoring_size():
+    """One linear of the scoring configuration at its full row count (64 x 768 = 49152 rows, 4096 x 4096 weight):
+    sampled rows against the oracle, row-permutation equivariance (a row's result does not depend on where in the
+    batch it sits: bit for bit), and rows of small integers against the exact integer product."""
+    m, n, k = 49152, 4096, 4096
+    q, s, q_d, s_d = _int8_case(n, k, seed=77)
+    gen = torch.Generator().manual_seed(78)
+    x = (torch.randn(4096, k, generator=gen) * 1.0).to(torch.bfloat16)
+    x = x.repeat(m // 4096, 1)                          # 12 copies of 4096 distinct rows
+    x[-3:] = torch.randint(-2, 3, (3, k), generator=gen).to(torch.bfloat16)   # exact rows at the very end
+    x_d = x.to(DEV)
+    y = ops.int8_mm_direct(x_d, q_d, s_d)
+    assert y.shape == (m, n) and bool(torch.isfinite(y.float()).all())
+    rows = [0, 1, 255, 256, 4095, 4096, 24575, 49151 - 3, 49151]
+    y_ref = qo.int8_linear_fp32(bf16_to_np(x[rows]), q, s)
+    assert qo.normwise_rel_err(bf16_to_np(y[rows].cpu()), y_ref) <= TOL
+    # copies of the same input row give the same output row wherever they sit
+    assert torch.equal(y[:4096], y[4096:8192]) and torch.equal(y[:4096], y[4096 * 5:4096 * 6])
+    perm = torch.randperm(m, generator=gen).to(DEV)
+    assert torch.equal(ops.int8_mm_direct(x_d[perm], q_d, s_d), y[perm])
+    y_int = qo.int8_linear_reference_rounding(bf16_to_np(x[-3:]), q, s)
+    assert np.array_equal(bf16_to_np(y[-3:].cpu()), y_int)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["int8", "int4"])
 def test_many_row_kernels_with_an_output_that_is_only_2_byte_aligned(mode):
     """The 32x32-tile kernels write 16-byte pieces of output rows; the C ABI only promises a 2-byte aligned y, so an
