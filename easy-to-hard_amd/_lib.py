@@ -27,6 +27,8 @@ _SIGNATURES = {
     "e2h_int4_dequantize_codes": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int, _P]),
     "e2h_int4_mm": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P, c_int64, _P]),
     "e2h_workspace_bytes": (c_int64, []),
+    "e2h_int4_mm_static_scratch": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P]),
+    "e2h_int4_mm_static_scratch_bytes": (c_int64, []),
     "e2h_decode_attention": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, _P]),
     "e2h_rmsnorm": (c_int, [_P, _P, _P, c_int64, c_int64, c_float, _P]),
     "e2h_add_rmsnorm": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),

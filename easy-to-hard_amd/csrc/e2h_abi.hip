@@ -23,6 +23,7 @@ extern "C" const char *e2h_status_string(int status) {
     case E2H_ERR_LAUNCH: return "HIP kernel launch failed";
     case E2H_ERR_NO_DEVICE: return "no gfx950 device";
     case E2H_ERR_BAD_OPTION: return "unknown option or value out of range";
+    case E2H_ERR_SCRATCH_TOO_SMALL: return "the call needs more scratch memory than the library's fixed buffer holds";
     default: return "unknown status";
   }
 }

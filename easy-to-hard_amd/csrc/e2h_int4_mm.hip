@@ -634,10 +634,14 @@ int launch_x_group_sums(const uint16_t *x, float *out, int M, int K, int stride,
 
 extern "C" int64_t e2h_workspace_bytes(void) { return static_cast<int64_t>(e2h::kTicketBytes) + (int64_t{32} << 20); }
 
-extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
-                           uint16_t *y, int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles,
-                           void *workspace, int64_t workspace_bytes, void *stream) {
-  using namespace e2h;
+namespace e2h {
+namespace {
+
+// strict_scratch: fail with E2H_ERR_SCRATCH_TOO_SMALL where the launch geometry chosen for the shape needs more scratch
+// than was passed, instead of falling back to a geometry that needs none
+int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y, int64_t m, int64_t n,
+                 int64_t k, int groupsize, int inner_k_tiles, void *workspace, int64_t workspace_bytes, void *stream,
+                 bool strict_scratch) {
   if (!x || !packed || !scales_and_zeros || !y) return E2H_ERR_NULL_POINTER;
   if (groupsize != 32 && groupsize != 64 && groupsize != 128 && groupsize != 256) return E2H_ERR_BAD_GROUPSIZE;
   if (inner_k_tiles != 2 && inner_k_tiles != 4 && inner_k_tiles != 8) return E2H_ERR_BAD_INNER_K_TILES;
@@ -698,7 +702,10 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     // workspace layout: [tickets | float partial tiles]
     const int64_t tile_floats = static_cast<int64_t>(sh.wn) * sh.t * mt * 4 * 64;
     const int64_t need = static_cast<int64_t>(kTicketBytes) + static_cast<int64_t>(n_blocks) * m_chunks * s * tile_floats * 4;
-    if (!have_ws || need > workspace_bytes || static_cast<int64_t>(n_blocks) * m_chunks * 4 > static_cast<int64_t>(kTicketBytes)) s = 1;
+    if (!have_ws || need > workspace_bytes || static_cast<int64_t>(n_blocks) * m_chunks * 4 > static_cast<int64_t>(kTicketBytes)) {
+      if (strict_scratch) return E2H_ERR_SCRATCH_TOO_SMALL;
+      s = 1;
+    }
   }
   a.S = s;
   a.ws_ticket = reinterpret_cast<unsigned *>(workspace);
@@ -754,6 +761,41 @@ extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint1
     if (rc != E2H_OK) return rc;
   }
   return E2H_OK;
+}
+
+// Scratch of the entry point that allocates nothing: split-K tickets followed by float32 partial tiles, the same layout
+// e2h_int4_mm expects of a caller's workspace.  Every GPU the library runs on holds its own copy until the process ends.
+constexpr size_t kStaticScratchBytes = kTicketBytes + (size_t{8} << 20);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, resolved on first use
+
+}  // namespace
+}  // namespace e2h
+
+extern "C" int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros,
+                           uint16_t *y, int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles,
+                           void *workspace, int64_t workspace_bytes, void *stream) {
+  return e2h::int4_mm_impl(x, packed, scales_and_zeros, y, m, n, k, groupsize, inner_k_tiles, workspace, workspace_bytes, stream, false);
+}
+
+extern "C" int64_t e2h_int4_mm_static_scratch_bytes(void) { return static_cast<int64_t>(e2h::kStaticScratchBytes); }
+
+extern "C" int e2h_int4_mm_static_scratch(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
+                                          int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *stream) {
+  using namespace e2h;
+  if (m > 64) return E2H_ERR_SCRATCH_TOO_SMALL;  // larger batches keep per-row group sums in scratch: outside the fixed budget
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return E2H_ERR_NO_DEVICE;
+  if (!g_scratch_ptr[dev]) {
+    // the array's name is a host-side handle, not a device address: resolve it once per device, with that device current.
+    // The array starts zeroed when the code object is loaded, and every launch leaves its tickets at zero again.
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return E2H_ERR_NO_DEVICE;
+    g_scratch_ptr[dev] = ptr;
+  }
+  return int4_mm_impl(x, packed, scales_and_zeros, y, m, n, k, groupsize, inner_k_tiles, g_scratch_ptr[dev],
+                      static_cast<int64_t>(kStaticScratchBytes), stream, true);
 }
 
 namespace e2h {

@@ -33,6 +33,7 @@ extern "C" {
 #define E2H_ERR_LAUNCH (-6)            /* the HIP runtime rejected the launch */
 #define E2H_ERR_NO_DEVICE (-7)         /* no gfx950 device is current */
 #define E2H_ERR_BAD_OPTION (-8)        /* unknown option name or value out of range */
+#define E2H_ERR_SCRATCH_TOO_SMALL (-9) /* the call needs more scratch than the fixed built-in buffer holds */
 
 /* Library identity / diagnostics (no reference counterpart). */
 int e2h_abi_version(void);
@@ -128,6 +129,19 @@ int e2h_int4_dequantize_codes(const int32_t *codes, const uint16_t *scales, cons
 int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
                 int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *workspace,
                 int64_t workspace_bytes, void *stream);
+
+/* e2h_int4_mm for callers that cannot allocate or pass scratch memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks and results (bit for
+ * bit) as e2h_int4_mm, but the split-K tickets and partial tiles live in a fixed buffer inside the library
+ * (e2h_int4_mm_static_scratch_bytes() = 64 KiB of tickets + 8 MiB of tiles, one copy per GPU, held until the process
+ * ends), and nothing is allocated or freed.  Limits: m <= 64 (decode batches); a shape whose launch geometry would need
+ * more scratch than the buffer holds returns E2H_ERR_SCRATCH_TOO_SMALL (no 7B / 34B linear at m <= 64 does).  All calls
+ * on one GPU share the buffer: calls that overlap on one GPU (two streams) race; order them on one stream.  The first
+ * call on a device resolves the buffer's device address (hipGetSymbolAddress); make that call before capturing a
+ * graph. */
+int e2h_int4_mm_static_scratch(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
+                               int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *stream);
+int64_t e2h_int4_mm_static_scratch_bytes(void);
 
 /* Gated feed-forward front half in one launch:  y = F.silu(w1(x)) * w3(x)  for two WeightOnlyInt4Linear
  * modules of equal shape (FeedForward.forward, reference models/model.py:343-344, with linear_forward_int4
