@@ -61,6 +61,9 @@ def parse_args():
                          "stock torch ops (what the reference's model code executes, without inductor); prints its own JSON line")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch-geometry override passed to e2h_set_option (experiments)")
+    ap.add_argument("--full-decode", action="store_true",
+                    help="run the whole decode of the configuration (every position once) and print its tok/s, as a check of "
+                         "the default mode's evenly spread sample of positions")
     ap.add_argument("--gemv-only", action="store_true",
                     help="only the back-to-back dequant-GEMV pass plus a 256 MiB calibration copy (for counter runs)")
     return ap.parse_args()
@@ -174,7 +177,7 @@ def stock_int4_operands(mod):
     return torch.ops.aten._convert_weight_to_int4pack(two_per_byte, mod.inner_k_tiles), mod.scales_and_zeros
 
 
-def measure_per_shape(model, rows_list, reps=6, stock=False):
+def measure_per_shape(model, rows_list, reps=6, stock=False, cpu=True):
     """Average launch duration of each distinct quantized-linear shape, replayed from a HIP graph and timed with events on
     the launch stream; the instances of a shape in different layers have different weights, so nothing stays cached."""
     import torch
@@ -230,57 +233,91 @@ def measure_per_shape(model, rows_list, reps=6, stock=False):
             if stock_ops is not None:
                 out[-1]["kernel"] = "aten._weight_int4pack_mm"
                 out[-1]["max_diff_vs_e2h"] = round(stock_err, 5)
+            if cpu:
+                # reference CPU path on the same shape: timed fully up to 64 rows, on a 512-row sample beyond
+                threads, _ = _cpu_threads()
+                torch.set_num_threads(threads)
+                rows = m if m <= 64 else min(m, 512)
+                cpu_s = _time_cpu(_cpu_case(mods[0], rows, torch.Generator().manual_seed(1234)), 1.0, max_runs=20) * (m / rows)
+                out[-1]["cpu_us"] = round(cpu_s * 1e6, 1)
+                out[-1]["cpu_threads"] = threads
+                out[-1]["cpu_rows_timed"] = rows
     return out
 
 
-def measure_cpu_baseline(model, batch, groupsize):
-    """Reference CPU path on the host cores: one layer's five linears + the LM head, extrapolated."""
+def _cpu_threads():
+    """Threads for the CPU baseline: the box's CPU share (OMP_NUM_THREADS where the scheduler sets it), else every
+    physical core.  Returns (threads used, physical cores of the host) -- both are reported."""
+    try:
+        import psutil
+
+        physical = psutil.cpu_count(logical=False) or os.cpu_count() or 1
+    except Exception:
+        physical = os.cpu_count() or 1
+    share = os.environ.get("OMP_NUM_THREADS")
+    threads = max(1, min(int(share), os.cpu_count() or 1)) if share and share.isdigit() else physical
+    return threads, physical
+
+
+def _time_cpu(fn, budget_s, max_runs=20):
+    """Median wall time of fn() after one warm-up run, repeated until the budget is used (at least twice)."""
+    fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 2 or (time.perf_counter() < t_end and len(times) < max_runs):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2]
+
+
+def _cpu_case(mod, rows, gen):
+    """Closure running the reference CPU path (dequantize + F.linear, oracle/reference_path.py) of one quantized linear
+    on `rows` rows of N(0, 1) bfloat16 activations."""
     import torch
 
     import easy_to_hard_amd as e2h
     from easy_to_hard_amd import ops
     from oracle import reference_path as rp
 
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-    torch.set_num_threads(cores)
-    backbone = model
+    x = torch.randn((rows, mod.in_features), generator=gen).to(torch.bfloat16)
+    if isinstance(mod, e2h.WeightOnlyInt4Linear):
+        codes = ops.int4_unpack(mod.weight).cpu()
+        sz = mod.scales_and_zeros.cpu()
+        g = mod.groupsize
+        return lambda: rp.int4_linear_cpu(x, codes, sz, g)
+    q, s = mod.weight.cpu(), mod.scales.cpu()
+    return lambda: rp.int8_linear_cpu(x, q, s)
+
+
+def measure_cpu_baseline(model, batch, groupsize, unit_rows=None, budget_s=2.5):
+    """Reference CPU path on the host cores: the quantized linears of one layer + the head at `batch` rows (decode), or at
+    a bounded sample of `unit_rows` rows (many-row passes), extrapolated to the whole step."""
+    import torch
+
+    threads, physical = _cpu_threads()
+    torch.set_num_threads(threads)
+    backbone = model.backbone if hasattr(model, "backbone") else model
     layer = backbone.layers[0]
     sample = [layer.attention.wqkv, layer.attention.wo, layer.feed_forward.w1, layer.feed_forward.w3, layer.feed_forward.w2]
     head = backbone.output
     gen = torch.Generator().manual_seed(1234)
-
-    def cpu_case(mod):
-        x = torch.randn((batch, mod.in_features), generator=gen).to(torch.bfloat16)
-        if isinstance(mod, e2h.WeightOnlyInt4Linear):
-            codes = ops.int4_unpack(mod.weight).cpu()
-            sz = mod.scales_and_zeros.cpu()
-            return lambda: rp.int4_linear_cpu(x, codes, sz, groupsize)
-        q, s = mod.weight.cpu(), mod.scales.cpu()
-        return lambda: rp.int8_linear_cpu(x, q, s)
-
-    def time_fn(fn, budget_s):
-        fn()
-        times = []
-        t_end = time.perf_counter() + budget_s
-        while len(times) < 2 or (time.perf_counter() < t_end and len(times) < 20):
-            t0 = time.perf_counter()
-            fn()
-            times.append(time.perf_counter() - t0)
-        times.sort()
-        return times[len(times) // 2]
-
-    layer_s = sum(time_fn(cpu_case(m), 2.5) for m in sample)
-    head_s = time_fn(cpu_case(head), 2.5)
+    rows = batch if unit_rows is None else min(unit_rows, batch)
+    layer_s = sum(_time_cpu(_cpu_case(m, rows, gen), budget_s) for m in sample)
+    head_s = _time_cpu(_cpu_case(head, rows, gen), budget_s)
     n_layer = len(backbone.layers)
-    step_s = layer_s * n_layer + head_s
+    step_s = (layer_s * n_layer + head_s) * (batch / rows)
     return {
         "value": round(batch / step_s, 3),
         "unit": "tok/s",
-        "cores": cores,
+        "cores": threads,
         "kind": "port",
-        "sample": f"quantized linears of 1 of {n_layer} layers + LM head at batch {batch} (dequantize + F.linear, torch CPU bf16), "
-                  f"median of repeated runs; layer {layer_s * 1e3:.1f} ms, head {head_s * 1e3:.1f} ms; extrapolated to a decode step "
-                  "(linears only, attention excluded)",
+        "sample": f"quantized linears of 1 of {n_layer} layers + head at {rows} rows"
+                  + (f" (a sample of the step's {batch} rows, scaled by {batch // rows})" if rows != batch else "")
+                  + f" (dequantize + F.linear, torch CPU bf16, {threads} threads; host has {physical} physical cores), "
+                  f"median of repeated runs; layer {layer_s * 1e3:.1f} ms, head {head_s * 1e3:.1f} ms; extrapolated to the whole "
+                  "step (linears only, attention excluded)",
     }
 
 
@@ -316,7 +353,7 @@ def run_reward_scoring(args, cfg, dev):
         "roofline": {"bound": "mfma", "achieved": round(flops * steps / elapsed / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": round(flops * steps / elapsed / 1e12 / 2500.0, 4), "traffic": None,
                      "note": "linear-layer flops over the whole step time (attention, norms and elementwise kernels included in the time)"},
-        "cpu_baseline": None,
+        "cpu_baseline": None if args.no_cpu_baseline else measure_cpu_baseline(model, batch * t, args.groupsize, unit_rows=2048, budget_s=1.0),
         "finite": bool(torch.isfinite(rewards.float()).all()),
     }))
 
@@ -355,8 +392,15 @@ def main():
     batch, t_prompt = args.batch, args.prompt
     if args.per_shape:
         rows_list = [int(v) for v in args.per_shape.split(",") if v]
-        print(json.dumps({"per_shape": measure_per_shape(model, rows_list, stock=args.stock), "model": args.model, "mode": args.mode,
-                          "groupsize": args.groupsize if args.mode == "int4" else None}))
+        rows_out = measure_per_shape(model, rows_list, stock=args.stock, cpu=not args.no_cpu_baseline)
+        cpu = None
+        if not args.no_cpu_baseline:
+            cpu = {"value": round(sum(r["cpu_us"] for r in rows_out), 1), "unit": "us (sum over the listed shapes and row counts)",
+                   "cores": rows_out[0]["cpu_threads"], "kind": "port",
+                   "sample": "dequantize + F.linear (torch CPU bf16) of every listed shape, median of repeated runs; row counts up to "
+                             "64 timed fully, larger ones on 512 rows and scaled (see cpu_rows_timed)"}
+        print(json.dumps({"per_shape": rows_out, "model": args.model, "mode": args.mode,
+                          "groupsize": args.groupsize if args.mode == "int4" else None, "cpu_baseline": cpu}))
         return
     if args.gemv_only:
         # counter-collection mode: the GEMV pass and a plain copy of known size (its FETCH_SIZE / WRITE_SIZE
@@ -381,7 +425,8 @@ def main():
                 mod.forward = (lambda x, w=w_stock, q=sz, g=mod.groupsize, n=mod.out_features:
                                torch.ops.aten._weight_int4pack_mm(x.reshape(-1, x.shape[-1]), w, g, q).reshape(*x.shape[:-1], n))
     max_seq = min(t_prompt + args.max_new, cfg.block_size)
-    assert args.warmup + args.steps < max_seq - t_prompt, "warmup + steps must fit in the decode budget"
+    n_new = max_seq - t_prompt
+    assert n_new >= 2, "the decode budget needs at least two new tokens"
     model.setup_caches(batch, max_seq)
     prompt = torch.randint(0, cfg.vocab_size, (batch, t_prompt), generator=torch.Generator().manual_seed(1234)).to(dev)
     input_pos = torch.arange(0, t_prompt, device=dev)
@@ -391,18 +436,53 @@ def main():
     prefill_s = time.time() - t0
     stepper = GraphedDecodeStep(model, batch, dev)
     cur = prefill(model, prompt, input_pos)  # the capture warm-up wrote cache row 0
-    pos = torch.tensor([t_prompt], device=dev, dtype=torch.int64)
+
+    if args.full_decode:
+        # the whole decode of the configuration, every position once, timed as the reference does
+        # (inference_generate.py:484-486: decoded tokens / wall time of decode_n_tokens)
+        pos = torch.tensor([t_prompt], device=dev, dtype=torch.int64)
+        for _ in range(args.warmup):
+            stepper.step(cur, pos)
+        cur = prefill(model, prompt, input_pos)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_new - 1):
+            cur = stepper.step(cur, pos)
+            pos += 1
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        print(json.dumps({"full_decode": True, "value": round(batch * (n_new - 1) / elapsed, 2), "unit": "tok/s",
+                          "ms_per_step": round(elapsed / (n_new - 1) * 1e3, 4), "steps": n_new - 1, "batch": batch,
+                          "prompt_len": t_prompt, "model": args.model, "mode": args.mode}))
+        return
+
+    # The timed steps sit at positions spread evenly over the whole decode (prompt .. prompt + new - 1), so that their
+    # average is the average step of the configuration whatever --steps is: decode attention reads every live cache
+    # position, so a step late in the decode costs more than one right after the prompt.  The graph reads the position
+    # from device memory; cache rows beyond the prompt hold N(0, 1) values standing in for the keys and values that the
+    # skipped steps would have written.
+    gen_dev = torch.Generator(device=dev).manual_seed(1234)
+    for blk in model.layers:
+        kv = blk.attention.kv_cache
+        for cache in (kv.k_cache, kv.v_cache):
+            cache[:, :, t_prompt:] = torch.randn(cache[:, :, t_prompt:].shape, generator=gen_dev, device=dev, dtype=torch.float32).to(cache.dtype)
+    steps = args.steps
+    positions = [t_prompt + (round(i * (n_new - 1) / (steps - 1)) if steps > 1 else (n_new - 1) // 2) for i in range(steps)]
+    pos_tensors = [torch.tensor([p], device=dev, dtype=torch.int64) for p in positions]
+    warm_pos = torch.tensor([t_prompt + (n_new - 1) // 2], device=dev, dtype=torch.int64)
     for _ in range(args.warmup):
-        cur = stepper.step(cur, pos).clone()
-        pos += 1
+        cur = stepper.step(cur, warm_pos).clone()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        cur = stepper.step(cur, pos)
-        pos += 1
+    for i in range(steps):
+        marks[i].record()
+        cur = stepper.step(cur, pos_tensors[i])
+    marks[steps].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    tok_s = batch * args.steps / elapsed
+    tok_s = batch * steps / elapsed
+    step_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
 
     if args.stock_step:
         print(json.dumps({"comparator": "stock torch ops + aten._weight_int4pack_mm, HIP-graph replayed decode step",
@@ -432,6 +512,9 @@ def main():
                         + f" weight-only linears, greedy decode, batch {batch}, prompt {t_prompt}, bf16 KV cache of {max_seq} positions, HIP-graph replayed decode step",
             "batch": batch,
             "prompt_len": t_prompt,
+            "new_tokens": n_new,
+            "timed_positions": f"{steps} steps at cache positions {positions[0]} .. {positions[-1]}, evenly spread over the decode",
+            "step_ms_first_mid_last": [round(step_ms[0], 4), round(step_ms[steps // 2], 4), round(step_ms[-1], 4)],
             "quantized_linears_per_step": roofline["launches_per_step"],
             "model_build_s": round(build_s, 2),
             "prefill_s": round(prefill_s, 3),

@@ -131,6 +131,50 @@ def generate(model, prompt: Tensor, max_new_tokens: int, use_graph: bool = True,
     return seq
 
 
+def load_model(checkpoint_path, device, precision=torch.bfloat16, use_tp: bool = False, model_name: Optional[str] = None):
+    """Counterpart of the reference's `_load_model` (inference_generate.py:224-259): the quantization mode is read off
+    the file name ("int8" / "int4" substrings, group size from the `.g{G}.` component), the module tree is built on the
+    meta device and converted by the matching QuantHandler, the state dict is memory-mapped with a weights-only load
+    and assigned, and the model moves to `device` in `precision` (integer buffers keep their dtype).
+
+    The architecture comes from the checkpoint's parent directory name, as in the reference, unless `model_name` names
+    it.  `use_tp` is accepted for signature compatibility; this build runs on one GPU and rejects it."""
+    from pathlib import Path
+
+    from .model import Transformer
+    from .quantize import WeightOnlyInt4QuantHandler, WeightOnlyInt8QuantHandler
+
+    if use_tp:
+        raise NotImplementedError("load_model: tensor parallelism is outside this one-GPU build")
+    checkpoint_path = Path(checkpoint_path)
+    if not checkpoint_path.is_file():
+        raise FileNotFoundError(str(checkpoint_path))
+    with torch.device("meta"):
+        model = Transformer.from_name(model_name if model_name is not None else checkpoint_path.parent.name)
+
+    if "int8" in str(checkpoint_path):
+        print("Using int8 weight-only quantization!")
+        model = WeightOnlyInt8QuantHandler(model).convert_for_runtime()
+
+    if "int4" in str(checkpoint_path):
+        print("Using int4 quantization!")
+        path_comps = checkpoint_path.name.split(".")
+        if len(path_comps) < 3 or not path_comps[-2].startswith("g") or not path_comps[-2][1:].isdigit():
+            raise ValueError(f"load_model: {checkpoint_path.name} names no group size (expected ...int4.g<G>.pth)")
+        groupsize = int(path_comps[-2][1:])
+        model = WeightOnlyInt4QuantHandler(model, groupsize).convert_for_runtime()
+
+    checkpoint = torch.load(str(checkpoint_path), mmap=True, weights_only=True)
+    expected = model.state_dict()
+    for key, want in expected.items():
+        if key in checkpoint and tuple(checkpoint[key].shape) != tuple(want.shape):
+            raise ValueError(f"load_model: {key} has shape {tuple(checkpoint[key].shape)} in {checkpoint_path.name}, "
+                             f"the model built for it expects {tuple(want.shape)}")
+    model.load_state_dict(checkpoint, assign=True)
+    model = model.to(device=device, dtype=precision)
+    return model.eval()
+
+
 @torch.no_grad()
 def model_score(reward_model, prompt: Tensor, max_seq_len: Optional[int] = None) -> Tensor:
     """Per-token rewards [B, T] of a RewardModel on a fully causal pass without KV cache."""

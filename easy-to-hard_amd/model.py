@@ -343,6 +343,9 @@ class Transformer(nn.Module):
                 mask = torch.logical_and(mask, visible[:, None, None, :])
                 mask = torch.logical_or(mask, self.self_mask[None, None, input_pos])
         freqs_cis = None if fused_step else self.freqs_cis[input_pos].to(dtype=x.dtype)
+        if fused_step and input_pos.dtype != torch.int64:
+            # the reference decodes with an int32 position tensor (inference_generate.py:205); the fused kernels read int64
+            input_pos = input_pos.to(torch.int64)
         if _fusable(x) and x.shape[-1] % 8 == 0 and self.norm.weight.dtype == torch.bfloat16:
             delta = None
             for layer in self.layers:

@@ -35,23 +35,61 @@ def _need_gpu(*tensors):
             )
 
 
-_workspaces = {}
+_workspaces = {}  # (device index, stream handle) -> scratch tensor; ("capture", device index) -> the one used under capture
+
+
+def _new_workspace(device):
+    return torch.zeros(int(_lib.load().e2h_workspace_bytes()), dtype=torch.uint8, device=device)
 
 
 def _workspace(device):
-    """One zero-initialised scratch tensor per device for the split-K tickets and partial tiles.  All launches
-    that use it are issued on the current stream, which orders them."""
-    ws = _workspaces.get(device.index)
+    """Zero-initialised scratch for the split-K tickets and partial tiles, one per (device, stream): launches on one
+    stream are ordered and may share it, launches on different streams must not (they would race on the tickets).
+
+    Work recorded into a HIP graph uses one further workspace per device, allocated eagerly together with the first
+    eager one: allocating it during capture would put it into the graph's private pool and record its zero fill
+    into the graph.  Graphs captured on one device therefore share scratch and must not replay concurrently."""
+    if torch.cuda.is_current_stream_capturing():
+        ws = _workspaces.get(("capture", device.index))
+        if ws is None:
+            raise RuntimeError(
+                "e2h: the first quantized-linear call on a device must run eagerly (it allocates the split-K scratch); "
+                "run one warm-up call before capturing a HIP graph"
+            )
+        return ws
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
     if ws is None:
-        ws = torch.zeros(int(_lib.load().e2h_workspace_bytes()), dtype=torch.uint8, device=device)
-        _workspaces[device.index] = ws
+        if ("capture", device.index) not in _workspaces:
+            _workspaces[("capture", device.index)] = _new_workspace(device)
+        ws = _new_workspace(device)
+        _workspaces[key] = ws
     return ws
 
 
+class _OnDevice:
+    """The library's entry points launch on the current device: calls for tensors of another device run under a
+    device guard (the caller's current device is left as it was)."""
+
+    def __init__(self, lib, device):
+        self._lib, self._device = lib, device
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        device = self._device
+
+        def call(*args):
+            with torch.cuda.device(device):
+                return fn(*args)
+
+        return call
+
+
 def _lib_for(t):
-    if t.device.index != torch.cuda.current_device():
-        torch.cuda.set_device(t.device)  # launches go to the current device's stream
-    return _lib.load()
+    lib = _lib.load()
+    if t.device.index == torch.cuda.current_device():
+        return lib
+    return _OnDevice(lib, t.device)
 
 
 # ---------------------------------------------------------------------------------------------

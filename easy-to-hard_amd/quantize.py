@@ -216,9 +216,11 @@ class WeightOnlyInt8Linear(torch.nn.Module):
         self.register_buffer("scales", torch.ones(out_features, dtype=torch.bfloat16))
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        # F.linear(input, self.weight.to(dtype=input.dtype)) * self.scales, as one kernel
+        # F.linear(input, self.weight.to(dtype=input.dtype)) * self.scales, as one kernel for bfloat16 activations
         if input.dtype != torch.bfloat16:
-            raise TypeError(f"WeightOnlyInt8Linear: bfloat16 activations expected, got {input.dtype}")
+            # float16 / float32 activations are outside the measured path: they run the reference's own two stock ops
+            # on the tensors' device (reference :428-429), with its dtype promotion (float16 * bfloat16 -> float32)
+            return F.linear(input, self.weight.to(dtype=input.dtype)) * self.scales
         x = input.reshape(-1, input.shape[-1])
         mm = torch.ops.e2h.int8_mm if torch.compiler.is_compiling() else ops.int8_mm_direct
         y = mm(x, self.weight, self.scales)

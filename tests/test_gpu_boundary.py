@@ -1,0 +1,157 @@
+"""GPU checks of the drop-in boundary: tracing under torch.compile(fullgraph=True) (the way the reference calls the
+modules in decode, inference_generate.py:346-349), the reference's int32 position tensor, per-stream split-K scratch,
+and the checkpoint writer -> file -> loader round trip (models/quantize.py:669-754, inference_generate.py:224-259)."""
+
+import pytest
+import torch
+
+import easy_to_hard_amd as e2h
+from easy_to_hard_amd import ops
+from easy_to_hard_amd.generate import GraphedDecodeStep, decode_one_token, generate, load_model, prefill
+from easy_to_hard_amd.model import Transformer, init_random_
+from tests.helpers import randn_bf16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tiny_int4(name="tiny-test", g=32):
+    model = Transformer.from_name(name)
+    init_random_(model, seed=1234, std=0.05)
+    sd = e2h.WeightOnlyInt4QuantHandler(model, groupsize=g).create_quantized_state_dict()
+    e2h.WeightOnlyInt4QuantHandler(model, groupsize=g).convert_for_runtime()
+    model.load_state_dict(sd, assign=True)
+    return model.to(device=DEV, dtype=torch.bfloat16).eval()
+
+
+def test_quantized_modules_trace_under_fullgraph_compile_and_match_eager():
+    """backend "aot_eager" traces with fake tensors through the registered e2h::int4_mm / e2h::int8_mm ops and then runs
+    the traced graph with the real kernels; fullgraph=True fails on any graph break."""
+    lin4 = e2h.WeightOnlyInt4Linear(512, 48, bias=False, groupsize=64, inner_k_tiles=8, padding=False).to(DEV)
+    w = randn_bf16((48, 512), std=0.02, seed=1).to(DEV)
+    lin4.weight, lin4.scales_and_zeros = e2h.prepare_int4_weight_and_scales_and_zeros(w, 64, 8)
+    lin8 = e2h.WeightOnlyInt8Linear(512, 48).to(DEV)
+    q, scales, _ = e2h.dynamically_quantize_per_channel(w.float(), -128, 127, torch.int8)
+    lin8.load_state_dict({"weight": q, "scales": scales})
+    x = randn_bf16((3, 5, 512), seed=2).to(DEV)
+    for lin in (lin4, lin8):
+        compiled = torch.compile(lin, backend="aot_eager", fullgraph=True)
+        with torch.no_grad():
+            assert torch.equal(compiled(x), lin(x))
+            assert torch.equal(compiled(x[:1, :1]), lin(x[:1, :1]))   # another shape retraces
+
+
+def test_decode_step_traces_under_fullgraph_compile():
+    """One decode step of a quantized model under torch.compile(fullgraph=True): the trace takes the stock-op branches
+    around the linears and the custom ops for the linears; logits agree with the eager fused step to bfloat16 noise and the
+    greedy token is the same."""
+    model = _tiny_int4()
+    bsz, t = 3, 9
+    model.setup_caches(bsz, 32)
+    prompt = torch.randint(0, model.config.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(5)).to(DEV)
+    pos = torch.arange(0, t, device=DEV)
+    with torch.no_grad():
+        cur = prefill(model, prompt, pos)
+        step_pos = torch.tensor([t], device=DEV)
+        eager = model(cur, step_pos).clone()
+        prefill(model, prompt, pos)
+        compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
+        traced = compiled(cur, step_pos)
+    err = (traced.float() - eager.float()).abs().max() / eager.float().abs().max()
+    assert err <= 2e-2, float(err)
+
+
+@pytest.mark.parametrize("name", ["tiny-test", "tiny-gqa-test"])
+def test_int32_position_tensor_as_the_reference_passes_it(name):
+    """The reference decodes with torch.tensor([T], dtype=torch.int) (inference_generate.py:205)."""
+    model = _tiny_int4(name, g=64)
+    bsz, t = 2, 8
+    model.setup_caches(bsz, 32)
+    prompt = torch.randint(0, model.config.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(3)).to(DEV)
+    pos = torch.arange(0, t, device=DEV)
+    cur = prefill(model, prompt, pos)
+    want = decode_one_token(model, cur, torch.tensor([t], device=DEV, dtype=torch.int64))
+    prefill(model, prompt, pos)
+    got = decode_one_token(model, cur, torch.tensor([t], device=DEV, dtype=torch.int))
+    assert torch.equal(got, want)
+    stepper = GraphedDecodeStep(model, bsz, DEV)
+    prefill(model, prompt, pos)
+    replay = stepper.step(cur, torch.tensor([t], device=DEV, dtype=torch.int)).clone()
+    assert torch.equal(replay, want)
+
+
+def test_two_streams_use_separate_split_k_scratch():
+    """Shapes that split K over workgroups (4096 x 4096 at 32 rows) issued concurrently on two streams: each stream has its
+    own tickets and partial tiles, and every result equals the single-stream one bit for bit."""
+    n, k, g = 4096, 4096, 128
+    w = randn_bf16((n, k), std=0.02, seed=9).to(DEV)
+    packed, sz = e2h.prepare_int4_weight_and_scales_and_zeros(w, g, 8)
+    q8, s8, _ = e2h.dynamically_quantize_per_channel(w.float(), -128, 127, torch.int8)
+    s8 = s8.to(torch.bfloat16)
+    xs = [randn_bf16((32, k), seed=20 + i).to(DEV) for i in range(2)]
+    want4 = [ops.int4_mm_direct(x, packed, g, sz) for x in xs]
+    want8 = [ops.int8_mm_direct(x, q8, s8) for x in xs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=DEV) for _ in range(2)]
+    got4, got8 = [[], []], [[], []]
+    for _ in range(40):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                got4[i].append(ops.int4_mm_direct(xs[i], packed, g, sz))
+                got8[i].append(ops.int8_mm_direct(xs[i], q8, s8))
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert all(torch.equal(y, want4[i]) for y in got4[i])
+        assert all(torch.equal(y, want8[i]) for y in got8[i])
+    keys = [key for key in ops._workspaces if key[0] == 0]
+    assert len({ops._workspaces[key].data_ptr() for key in keys}) >= 3   # default stream + the two side streams
+
+
+@pytest.mark.parametrize("mode,g", [("int4", 64), ("int8", 128)])
+def test_writer_file_loader_round_trip(tmp_path, mode, g):
+    """quantize() writes model{label}int4.g{G}.pth / model{label}int8.pth next to model.pth; load_model() reads the mode and
+    the group size off that name, builds the module tree from the directory name, and the loaded model decodes exactly
+    like one converted in memory."""
+    ckpt_dir = tmp_path / "tiny-gqa-test"
+    ckpt_dir.mkdir()
+    model = Transformer.from_name("tiny-gqa-test")
+    init_random_(model, seed=1234, std=0.05)
+    torch.save(model.state_dict(), ckpt_dir / "model.pth")
+    out = e2h.quantize(ckpt_dir / "model.pth", mode, g, "_")
+    assert out.name == ("model_int4.g64.pth" if mode == "int4" else "model_int8.pth")
+    loaded = load_model(out, DEV, torch.bfloat16, use_tp=False)
+    lin = loaded.layers[0].attention.wqkv
+    if mode == "int4":
+        assert isinstance(lin, e2h.WeightOnlyInt4Linear) and lin.groupsize == g and lin.weight.dtype == torch.int32 and lin.weight.is_cuda
+        handler = e2h.WeightOnlyInt4QuantHandler(model, groupsize=g)
+    else:
+        assert isinstance(lin, e2h.WeightOnlyInt8Linear) and lin.weight.dtype == torch.int8 and lin.scales.dtype == torch.bfloat16
+        handler = e2h.WeightOnlyInt8QuantHandler(model)
+    assert loaded.tok_embeddings.weight.dtype == torch.bfloat16 and not loaded.training
+    sd = handler.create_quantized_state_dict()
+    handler.convert_for_runtime()
+    model.load_state_dict(sd, assign=True)
+    model = model.to(device=DEV, dtype=torch.bfloat16).eval()
+    prompt = torch.randint(0, model.config.vocab_size, (2, 6), generator=torch.Generator().manual_seed(8)).to(DEV)
+    assert torch.equal(generate(loaded, prompt, 5, use_graph=False), generate(model, prompt, 5, use_graph=False))
+
+
+def test_loader_rejects_what_it_cannot_interpret(tmp_path):
+    ckpt_dir = tmp_path / "tiny-test"
+    ckpt_dir.mkdir()
+    model = Transformer.from_name("tiny-test")
+    init_random_(model, seed=1, std=0.05)
+    torch.save(model.state_dict(), ckpt_dir / "model.pth")
+    out = e2h.quantize(ckpt_dir / "model.pth", "int4", 64, "")
+    bad = ckpt_dir / "modelint4.pth"          # no .g{G}. component
+    out.rename(bad)
+    with pytest.raises(ValueError):
+        load_model(bad, DEV)
+    wrong = ckpt_dir / "modelint4.g128.pth"   # group size in the name differs from the tensors' shapes
+    bad.rename(wrong)
+    with pytest.raises(ValueError):
+        load_model(wrong, DEV)
+    with pytest.raises(FileNotFoundError):
+        load_model(ckpt_dir / "missing_int8.pth", DEV)
+    with pytest.raises(NotImplementedError):
+        load_model(wrong, DEV, use_tp=True)

@@ -10,7 +10,7 @@ import torch
 import torch.nn as nn
 
 import easy_to_hard_amd as e2h
-from easy_to_hard_amd.generate import GraphedDecodeStep, decode_one_token, generate, model_score, prefill
+from easy_to_hard_amd.generate import GraphedDecodeStep, decode_one_token, generate, load_model, model_score, prefill
 from easy_to_hard_amd.model import ModelArgs, RewardModel, Transformer, init_random_
 from oracle import quant_oracle as qo
 from tests.helpers import bf16_to_np
@@ -62,12 +62,8 @@ def test_int4_checkpoint_roundtrip_and_greedy_decode(tmp_path, name, g):
     assert sd["layers.0.attention.wqkv.weight"].dtype == torch.int32
     assert sd["output.scales_and_zeros"].shape == (model.config.dim // g, model.config.vocab_size, 2)
 
-    # runtime path of the reference loader: swap modules on the meta device, load, move to the GPU
-    with torch.device("meta"):
-        rt = Transformer.from_name(name)
-    e2h.WeightOnlyInt4QuantHandler(rt, groupsize=int(path.name.split(".")[-2][1:])).convert_for_runtime()
-    rt.load_state_dict(torch.load(path, mmap=True, weights_only=True), assign=True)
-    rt = rt.to(device=DEV, dtype=torch.bfloat16).eval()
+    # runtime path of the reference loader (inference_generate.py:224-259)
+    rt = load_model(path, DEV, torch.bfloat16, model_name=name)
     assert rt.output.weight.dtype == torch.int32 and rt.output.weight.is_cuda
 
     oracle = _oracle_copy(rt, "int4", g)
