@@ -42,12 +42,19 @@ Pinning status (what independent evidence each restatement is checked against in
                               pinned: float64 brute force on tiny cases and the library kernels
                               torch.ops.aten._weight_int8pack_mm and
                               aten._convert_weight_to_int4pack_for_cpu/_weight_int4pack_mm_for_cpu.
-  int4_tile_pack              PARITY UNPINNED against PyTorch 2.2.0's CUDA kernel: that source is not
-                              in the reference tree or this image and the reference holds no packed
-                              checkpoint.  The nibble order below is the published algorithm of
-                              `matrix_to_m16n8k16_Bint4_layout`; tests pin self-consistency only
-                              (brute-force scalar packer, unpack(pack(q)) == q, and end-to-end matmul
-                              agreement, which fails loudly if pack and matmul disagree on the order).
+  int4_tile_pack              word format pinned on the GPU against PyTorch-ROCm's own
+                              aten._convert_weight_to_int4pack (an independent library with the same bit
+                              formula inside a word and another lane map): every checkpoint word is a fixed
+                              gather of nibbles from two of that packer's words and must equal this function's
+                              output bit for bit (tests/test_gpu_configs_at_size.py).  That pins the nibble
+                              order inside a word, the pairing of two 16-wide k tiles per word and the outer
+                              [N tile][K super-tile][lane][pair] order.
+                              PARITY UNPINNED: the lane map of the PyTorch 2.2.0 CUDA kernel itself (lane t holds
+                              row 8 * nTile + t / 4 and k = 2j, 2j+1, 2j+8, 2j+9 with j = t % 4).  That source
+                              (`matrix_to_m16n8k16_Bint4_layout`) is not in the reference tree or this image and
+                              the reference holds no packed checkpoint; the published algorithm is restated
+                              and the CPU tests pin self-consistency only (brute-force scalar packer,
+                              unpack(pack(q)) == q, end-to-end matmul agreement).
 """
 
 import numpy as np
