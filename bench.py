@@ -2,16 +2,19 @@
 """Benchmark of the quantized-linear hot path on one MI355X.
 
 Workload (default): BASELINE config "random-init Llama-2-7B-architecture model with int4 g128 weight-only
-linears, batch 32, prompt 256, greedy decode, bf16 KV cache".  One step = one decode step of the whole batch
-(129 dequant-GEMV launches -- w1 and w3 of a block share one gated launch -- plus decode attention, norms, RoPE), replayed from a HIP graph.  `value` is decoded
-tokens per second = batch * steps / time, with everything resident in HBM.
+linears, batch 32, prompt 256, 512 greedy-decoded tokens, bf16 KV cache".  One step = one decode step of the whole
+batch (129 dequant-GEMV launches -- w1 and w3 of a block share one gated launch -- plus decode attention, norms,
+RoPE), replayed from a HIP graph.  The timed steps sit at cache positions spread evenly over the whole decode, so
+`value` -- decoded tokens per second = batch * steps / time, everything resident in HBM -- is the configuration's
+average whatever --steps is (--full-decode runs every position once as a check).
 
 Extra objects on the JSON line:
   roofline      the dequant-GEMV kernels of one decode step launched back to back (all of them, each on its
                 own weights, 3.5 GB working set per pass so no cache holds it), timed with events on the
                 launch stream: algorithmic bytes / average launch duration against 8 TB/s.
   cpu_baseline  the reference CPU path (dequantize + F.linear, torch CPU ops) on the host cores for one
-                transformer layer + LM head at the same batch, extrapolated to a full decode step.
+                transformer layer + LM head at the same batch, extrapolated to a full decode step (every other mode
+                -- --per-shape, --reward, --model 34B, --mode int8 -- carries its own CPU leg).
 """
 
 import argparse
