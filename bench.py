@@ -72,6 +72,14 @@ def parse_args():
     return ap.parse_args()
 
 
+def spread_positions(t_prompt, n_new, steps):
+    """Cache positions of the timed decode steps: `steps` positions spread evenly over t_prompt .. t_prompt + n_new - 1
+    (both ends included; a single step sits in the middle), so that their mean is the mean position of the decode."""
+    if steps <= 1:
+        return [t_prompt + (n_new - 1) // 2] * max(steps, 0)
+    return [t_prompt + round(i * (n_new - 1) / (steps - 1)) for i in range(steps)]
+
+
 def quantized_linears(model):
     import easy_to_hard_amd as e2h
 
@@ -470,7 +478,7 @@ def main():
         for cache in (kv.k_cache, kv.v_cache):
             cache[:, :, t_prompt:] = torch.randn(cache[:, :, t_prompt:].shape, generator=gen_dev, device=dev, dtype=torch.float32).to(cache.dtype)
     steps = args.steps
-    positions = [t_prompt + (round(i * (n_new - 1) / (steps - 1)) if steps > 1 else (n_new - 1) // 2) for i in range(steps)]
+    positions = spread_positions(t_prompt, n_new, steps)
     pos_tensors = [torch.tensor([p], device=dev, dtype=torch.int64) for p in positions]
     warm_pos = torch.tensor([t_prompt + (n_new - 1) // 2], device=dev, dtype=torch.int64)
     for _ in range(args.warmup):

@@ -242,3 +242,41 @@ def test_bench_refuses_more_than_one_gpu():
 
     proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert proc.returncode == 2 and "one GPU" in proc.stderr
+
+
+def test_bench_spreads_the_timed_positions_over_the_whole_decode():
+    import bench
+
+    pos = bench.spread_positions(256, 512, 20)
+    assert len(pos) == 20 and pos[0] == 256 and pos[-1] == 767 and pos == sorted(pos)
+    assert abs(sum(pos) / len(pos) - (256 + 767) / 2) < 1.0          # the sample's mean position is the decode's
+    assert bench.spread_positions(256, 512, 511 + 1)[:3] == [256, 257, 258]
+    assert bench.spread_positions(10, 5, 1) == [12] and bench.spread_positions(10, 5, 2) == [10, 14]
+    threads, physical = bench._cpu_threads()
+    assert threads >= 1 and physical >= 1
+
+
+def test_loader_reads_mode_and_group_size_off_the_file_name(tmp_path):
+    """load_model (the reference's _load_model, inference_generate.py:224-259): a plain bf16 checkpoint loads on the CPU;
+    names it cannot interpret and missing files are refused before anything touches a GPU."""
+    import torch
+
+    from easy_to_hard_amd.generate import load_model
+    from easy_to_hard_amd.model import Transformer, init_random_
+
+    ckpt_dir = tmp_path / "tiny-test"
+    ckpt_dir.mkdir()
+    model = Transformer.from_name("tiny-test")
+    init_random_(model, seed=3, std=0.05)
+    torch.save(model.state_dict(), ckpt_dir / "model.pth")
+    loaded = load_model(ckpt_dir / "model.pth", "cpu", torch.bfloat16)
+    assert not loaded.training and loaded.output.weight.dtype == torch.bfloat16
+    assert torch.equal(loaded.output.weight, model.output.weight.to(torch.bfloat16))
+    assert torch.equal(loaded.layers[1].attention.wqkv.weight, model.layers[1].attention.wqkv.weight.to(torch.bfloat16))
+    (ckpt_dir / "model_int4.pth").write_bytes(b"x")                     # "int4" but no .g{G}. component
+    with pytest.raises(ValueError):
+        load_model(ckpt_dir / "model_int4.pth", "cpu")
+    with pytest.raises(FileNotFoundError):
+        load_model(ckpt_dir / "absent_int8.pth", "cpu")
+    with pytest.raises(NotImplementedError):
+        load_model(ckpt_dir / "model.pth", "cpu", use_tp=True)
