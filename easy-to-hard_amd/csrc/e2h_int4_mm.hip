@@ -115,7 +115,6 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     uint16_t *__restrict__ y, float *__restrict__ ws_partial, unsigned *__restrict__ ws_ticket, int M, int N, int K,
     int slabs_in_x, RopeArgs rope, const float *__restrict__ xsum, int xsum_stride) {
   constexpr bool GATE = EPI == kGate;
-  static_assert(EPI != kRope || T == 1, "the rotary epilogue handles one column tile per wave");
   static_assert(!GATE || T == 2, "gate mode pairs exactly two weight matrices");
   constexpr int TC = GATE ? 1 : T;  // distinct column tiles per wave
   typedef Int4Geom<G, IKT> Geo;
@@ -352,7 +351,12 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   wregs_t ring[NB];
   u32x4_t xstage[XD][kPiecesPerThread];
   int rope_pos = -1;
-  float rope_cs = 1.f, rope_sn = 0.f;
+  float rope_cs[TC], rope_sn[TC];
+#pragma unroll
+  for (int t = 0; t < TC; ++t) {
+    rope_cs[t] = 1.f;
+    rope_sn[t] = 0.f;
+  }
   if (C1 > C0) {
 #pragma unroll
     for (int d = 0; d < XD; ++d) load_x(xstage[d], d);
@@ -362,11 +366,14 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
       // the rotation's cos / sin depend on a position read from memory: fetch both now, behind the first
       // weight loads, instead of as two dependent round trips at the very end
       rope_pos = static_cast<int>(rope.input_pos[0]);
-      const int ncol = 16 * tile16_0 + c;
-      if (ncol < N && rope_pos >= 0 && rope_pos < rope.S && ncol < (rope.H + rope.Hkv) * rope.D) {
-        const uint32_t f = reinterpret_cast<const uint32_t *>(rope.freqs)[static_cast<size_t>(rope_pos) * (rope.D / 2) + ((ncol % rope.D) >> 1)];
-        rope_cs = __builtin_bit_cast(float, f << 16);
-        rope_sn = __builtin_bit_cast(float, f & 0xFFFF0000u);
+#pragma unroll
+      for (int t = 0; t < TC; ++t) {
+        const int ncol = 16 * (tile16_0 + t) + c;
+        if (ncol < N && rope_pos >= 0 && rope_pos < rope.S && ncol < (rope.H + rope.Hkv) * rope.D) {
+          const uint32_t f = reinterpret_cast<const uint32_t *>(rope.freqs)[static_cast<size_t>(rope_pos) * (rope.D / 2) + ((ncol % rope.D) >> 1)];
+          rope_cs[t] = __builtin_bit_cast(float, f << 16);
+          rope_sn[t] = __builtin_bit_cast(float, f & 0xFFFF0000u);
+        }
       }
     }
     store_x(xstage[0], 0);
@@ -462,34 +469,37 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
   }
   if (kg != 0) return;
   if constexpr (EPI == kRope) {
-    const int n = 16 * tile16_0 + c;
     const int D = rope.D, H = rope.H, Hkv = rope.Hkv;
-    const int head = n / D, d = n % D;
     const int pos = rope_pos;
-    const bool in_range = n < N && pos >= 0 && pos < rope.S;
-    const bool rotated = head < H + Hkv;
-    const float cs = rope_cs, sn = rope_sn;
-    uint16_t *dst;  // element (m = 0) of this lane's column; rows are row_stride apart
-    size_t row_stride;
-    if (head < H) {
-      dst = rope.q_out + static_cast<size_t>(head) * D + d;
-      row_stride = static_cast<size_t>(H) * D;
-    } else {
-      const int hk = rotated ? head - H : head - H - Hkv;
-      dst = (rotated ? rope.kc : rope.vc) + (static_cast<size_t>(hk) * rope.S + pos) * D + d;
-      row_stride = static_cast<size_t>(Hkv) * rope.S * D;
-    }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int m = m_base + 16 * mt + 4 * b + q;
-        const float own = bf16_round(acc[0][mt][q]);
-        const float other = __shfl_xor(own, 1);  // the pair's other column lives in the neighbouring lane
-        // even column: x0 * cos - x1 * sin; odd column: x1 * cos + x0 * sin (two rounded products, then the sum)
-        const float r = (c & 1) ? own * cs + other * sn : own * cs - other * sn;
-        if (in_range && m < M) dst[static_cast<size_t>(m) * row_stride] = f32_to_bf16_rne(rotated ? r : own);
+    for (int t = 0; t < TC; ++t) {
+      const int n = 16 * (tile16_0 + t) + c;
+      const int head = n / D, d = n % D;
+      const bool in_range = n < N && pos >= 0 && pos < rope.S;
+      const bool rotated = head < H + Hkv;
+      const float cs = rope_cs[t], sn = rope_sn[t];
+      uint16_t *dst;  // element (m = 0) of this lane's column; rows are row_stride apart
+      size_t row_stride;
+      if (head < H) {
+        dst = rope.q_out + static_cast<size_t>(head) * D + d;
+        row_stride = static_cast<size_t>(H) * D;
+      } else {
+        const int hk = rotated ? head - H : head - H - Hkv;
+        dst = (rotated ? rope.kc : rope.vc) + (static_cast<size_t>(hk) * rope.S + pos) * D + d;
+        row_stride = static_cast<size_t>(Hkv) * rope.S * D;
       }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int m = m_base + 16 * mt + 4 * b + q;
+          const float own = bf16_round(acc[t][mt][q]);
+          const float other = __shfl_xor(own, 1);  // the pair's other column lives in the neighbouring lane
+          // even column: x0 * cos - x1 * sin; odd column: x1 * cos + x0 * sin (two rounded products, then the sum)
+          const float r = (c & 1) ? own * cs + other * sn : own * cs - other * sn;
+          if (in_range && m < M) dst[static_cast<size_t>(m) * row_stride] = f32_to_bf16_rne(rotated ? r : own);
+        }
+    }
     return;
   }
   if constexpr (GATE) {
@@ -682,6 +692,11 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
     const int blocks = ((tiles16 + 3) / 4) * m_chunks;
     if (have_ws)
       while (s < 4 && blocks * s * 2 <= kCUs && nchunks / (2 * s * sh.wk) >= 4) s *= 2;
+    // More column blocks than CUs: a wave with two column tiles takes about 1.5x as long as with one, and halving the
+    // number of workgroups saves more than that whenever one tile per wave needs a second round of workgroups
+    // (measured: 10240 x 8192 at 64 rows 32.9 instead of 44.5 us, 32000 x 8192 71.5 instead of 97.7,
+    // 32000 x 4096 at 32 rows 24.8 instead of 27.2; with 16-row workgroups one tile per wave stays ahead)
+    if (mt == 2 && blocks > kCUs) sh.t = 2;
   } else if (wide_ok) {
     // many rows of x (prefill, scoring): every weight fragment feeds four row tiles straight from registers;
     // wide column blocks keep the LDS traffic for activation fragments below the MFMA rate
@@ -889,9 +904,14 @@ extern "C" int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, con
   a.S = 1; a.ws_partial = nullptr; a.ws_ticket = nullptr; a.xsum = nullptr; a.xsum_stride = 0;
   a.stream = static_cast<hipStream_t>(stream);
   const bool two = a.M > 16;
+  // 32-row workgroups: two column tiles per wave once one tile per wave would need more workgroups than CUs
+  // (as in e2h_int4_mm; batches of 33 .. 64 rows run two row slabs per column block)
+  const int tiles16 = (a.N + 15) / 16;
+  const int opt_t = options().int4_rows_per_wave / 16;
+  const bool wide = two && (opt_t ? opt_t == 2 : ((tiles16 + 3) / 4) * ((a.M + 31) / 32) > kCUs);
   switch (groupsize) {
-    case 32: return two ? launch<32, 8, 2, 1, 4, 2, kRope>(a) : launch<32, 8, 1, 1, 4, 2, kRope>(a);
-    case 64: return two ? launch<64, 8, 2, 1, 4, 2, kRope>(a) : launch<64, 8, 1, 1, 4, 2, kRope>(a);
-    default: return two ? launch<128, 8, 2, 1, 4, 2, kRope>(a) : launch<128, 8, 1, 1, 4, 2, kRope>(a);
+    case 32: return wide ? launch<32, 8, 2, 2, 4, 2, kRope>(a) : two ? launch<32, 8, 2, 1, 4, 2, kRope>(a) : launch<32, 8, 1, 1, 4, 2, kRope>(a);
+    case 64: return wide ? launch<64, 8, 2, 2, 4, 2, kRope>(a) : two ? launch<64, 8, 2, 1, 4, 2, kRope>(a) : launch<64, 8, 1, 1, 4, 2, kRope>(a);
+    default: return wide ? launch<128, 8, 2, 2, 4, 2, kRope>(a) : two ? launch<128, 8, 2, 1, 4, 2, kRope>(a) : launch<128, 8, 1, 1, 4, 2, kRope>(a);
   }
 }

@@ -263,8 +263,11 @@ def test_34b_gated_pair_2x22016x8192_g64(m):
     assert torch.equal(y, ops.silu_mul(ya, yb))
 
 
-def test_34b_grouped_query_projection_with_rope_and_cache_write_g64():
-    bsz, n_head, n_kv, d, k, g = 64, 64, 8, 128, 8192, 64
+@pytest.mark.parametrize("bsz,tiles_per_wave", [(64, 0), (64, 1), (33, 2), (32, 0), (32, 2)])
+def test_34b_grouped_query_projection_with_rope_and_cache_write_g64(bsz, tiles_per_wave):
+    """tiles_per_wave 0 = the library's own choice (two column tiles per wave at 33 .. 64 rows of this shape, one at 32),
+    1 / 2 = that geometry forced for the fused launch."""
+    n_head, n_kv, d, k, g = 64, 8, 128, 8192, 64
     n = (n_head + 2 * n_kv) * d
     s_max, pos = 96, 41
     packed, sz = _big_int4_weight(n, k, g, seed=3)
@@ -276,7 +279,11 @@ def test_34b_grouped_query_projection_with_rope_and_cache_write_g64():
     freqs = precompute_freqs_cis(s_max, d, 1000000, device=DEV)
     input_pos = torch.tensor([pos], device=DEV)
     kc, vc = kc0.clone(), vc0.clone()
-    q = ops.int4_mm_rope_kv(xd, packed, sz, g, freqs, kc, vc, input_pos, n_head, n_kv, d)
+    _lib.set_option("int4_rows_per_wave", 16 * tiles_per_wave)
+    try:
+        q = ops.int4_mm_rope_kv(xd, packed, sz, g, freqs, kc, vc, input_pos, n_head, n_kv, d)
+    finally:
+        _lib.set_option("int4_rows_per_wave", 0)
     _lib.set_option("int4_k_slices", 1)
     try:
         qkv = ops.int4_mm_direct(xd, packed, g, sz)
