@@ -30,6 +30,8 @@
 // several chunks ahead in registers.  With S > 1 the slices meet in a workspace: each workgroup stores its
 // float32 partial tile, takes a ticket, and the last one to arrive adds the S partials in slice order -- a
 // fixed order, so results are deterministic -- and writes bf16.
+#include <atomic>
+
 #include "e2h_common.h"
 #include "e2h_int4_unpack.h"
 
@@ -783,7 +785,9 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
 constexpr size_t kStaticScratchBytes = kTicketBytes + (size_t{8} << 20);
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
-void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, resolved on first use
+// device address of `scratch` on each device, resolved on first use (host threads may race to resolve it: they store
+// the same value)
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
 
 }  // namespace
 }  // namespace e2h
@@ -802,14 +806,16 @@ extern "C" int e2h_int4_mm_static_scratch(const uint16_t *x, const int32_t *pack
   if (m > 64) return E2H_ERR_SCRATCH_TOO_SMALL;  // larger batches keep per-row group sums in scratch: outside the fixed budget
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return E2H_ERR_NO_DEVICE;
-  if (!g_scratch_ptr[dev]) {
+  void *scratch_ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!scratch_ptr) {
     // the array's name is a host-side handle, not a device address: resolve it once per device, with that device current.
     // The array starts zeroed when the code object is loaded, and every launch leaves its tickets at zero again.
     void *ptr = nullptr;
     if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return E2H_ERR_NO_DEVICE;
-    g_scratch_ptr[dev] = ptr;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    scratch_ptr = ptr;
   }
-  return int4_mm_impl(x, packed, scales_and_zeros, y, m, n, k, groupsize, inner_k_tiles, g_scratch_ptr[dev],
+  return int4_mm_impl(x, packed, scales_and_zeros, y, m, n, k, groupsize, inner_k_tiles, scratch_ptr,
                       static_cast<int64_t>(kStaticScratchBytes), stream, true);
 }
 
