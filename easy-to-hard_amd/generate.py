@@ -175,6 +175,42 @@ def load_model(checkpoint_path, device, precision=torch.bfloat16, use_tp: bool =
     return model.eval()
 
 
+def load_reward_model(checkpoint_path, device, precision=torch.bfloat16, use_tp: bool = False,
+                      model_name: Optional[str] = None, on_the_fly_8bit_quantization: bool = False):
+    """Counterpart of the reference's `_load_reward_model` (inference_reward.py:94-118) and of the quantization step
+    its `main` runs afterwards (:171-178): the checkpoint is a bfloat16 language-model state dict (quantized files are
+    rejected, as there), loaded memory-mapped into the backbone built on the meta device; the `output` projection becomes
+    the zero-initialised two-row score head (a fine-tuned head is loaded over it by the caller); the model moves to
+    `device` in `precision`; with `on_the_fly_8bit_quantization` every linear, head included, is then quantized to int8
+    per channel on the device by `WeightOnlyInt8QuantHandler.convert_for_runtime_on_the_fly`."""
+    from pathlib import Path
+
+    from .model import ModelArgs, RewardModel, Transformer, apply_reward_modeling_head
+    from .quantize import WeightOnlyInt8QuantHandler
+
+    if use_tp:
+        raise NotImplementedError("load_reward_model: tensor parallelism is outside this one-GPU build")
+    checkpoint_path = Path(checkpoint_path)
+    if "int8" in str(checkpoint_path):
+        raise NotImplementedError("int8 quantization cannot be used for reward model!")
+    if "int4" in str(checkpoint_path):
+        raise NotImplementedError("int4 quantization cannot be used for reward model!")
+    if not checkpoint_path.is_file():
+        raise FileNotFoundError(str(checkpoint_path))
+    config = ModelArgs.from_name(model_name if model_name is not None else checkpoint_path.parent.name)
+    with torch.device("meta"):
+        model = RewardModel(config)
+        model.backbone = Transformer(config)  # full vocabulary projection, as in the language-model checkpoint
+    checkpoint = torch.load(str(checkpoint_path), mmap=True, weights_only=True)
+    model.backbone.load_state_dict(checkpoint, assign=True)
+    apply_reward_modeling_head(model.backbone)
+    model = model.to(device=device, dtype=precision).eval()
+    if on_the_fly_8bit_quantization:
+        model = WeightOnlyInt8QuantHandler(model).convert_for_runtime_on_the_fly()
+        model = model.to(device=device).eval()
+    return model
+
+
 @torch.no_grad()
 def model_score(reward_model, prompt: Tensor, max_seq_len: Optional[int] = None) -> Tensor:
     """Per-token rewards [B, T] of a RewardModel on a fully causal pass without KV cache."""

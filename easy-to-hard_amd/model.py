@@ -373,6 +373,39 @@ class RewardModel(nn.Module):
             rewards = rewards.gather(dim=-1, index=eos_pos.unsqueeze(-1)).squeeze(-1)
         return rewards
 
+    @property
+    def backbone_model(self) -> "Transformer":
+        """The reference's name for the backbone (models/reward_model.py:72)."""
+        return self.backbone
+
+    @classmethod
+    def from_name(cls, name: str, head_rows: int = 2) -> "RewardModel":
+        return cls(ModelArgs.from_name(name), head_rows)
+
+
+def apply_reward_modeling_head(transformer: "Transformer", requires_grad: bool = False, init_scheme: str = "zeros") -> None:
+    """Turn a language model's `output` projection into the two-row score head, in place (reference
+    models/reward_model.py:95-133): "zeros" starts from a zero head, "semantic" from the rows of the tokens "2" (id 29906)
+    and, negated, "1" (id 29896) of the existing projection, "random" from a Kaiming-uniform draw (seed 42) scaled by
+    sqrt(2).  The head keeps the dtype and device of the projection it replaces."""
+    import math
+
+    out = transformer.output
+    old = out.weight
+    head = torch.zeros((2, old.shape[1]), dtype=old.dtype, device=old.device)
+    if init_scheme == "semantic":
+        with torch.no_grad():
+            head[0] = old[29906]
+            head[1] = -old[29896]
+    elif init_scheme == "random":
+        gen = torch.Generator(device=head.device).manual_seed(42)
+        nn.init.kaiming_uniform_(head, a=math.sqrt(5), generator=gen)
+        head = head * math.sqrt(2.0)
+    elif init_scheme != "zeros":
+        raise ValueError(f"Unknown init_scheme: {init_scheme}")
+    out.weight = nn.Parameter(head, requires_grad=requires_grad)
+    out.out_features = 2
+
 
 def init_random_(model: nn.Module, seed: int = 1234, std: float = 0.02, device=None) -> nn.Module:
     """Random-init every linear and the embedding with N(0, std), norms with ones, in bfloat16.

@@ -280,3 +280,43 @@ def test_loader_reads_mode_and_group_size_off_the_file_name(tmp_path):
         load_model(ckpt_dir / "absent_int8.pth", "cpu")
     with pytest.raises(NotImplementedError):
         load_model(ckpt_dir / "model.pth", "cpu", use_tp=True)
+
+
+def test_reward_model_loader_builds_the_two_row_head_and_rejects_quantized_files(tmp_path):
+    """load_reward_model follows the reference's _load_reward_model (inference_reward.py:94-118): a bfloat16
+    language-model checkpoint goes into the backbone, `output` becomes a zero two-row head, quantized file names are
+    refused; apply_reward_modeling_head covers the three initialisations of models/reward_model.py:95-133."""
+    from easy_to_hard_amd.generate import load_reward_model
+    from easy_to_hard_amd.model import RewardModel, apply_reward_modeling_head, init_random_
+
+    ckpt_dir = tmp_path / "tiny-test"
+    ckpt_dir.mkdir()
+    lm = Transformer.from_name("tiny-test")
+    init_random_(lm, seed=3, std=0.05)
+    torch.save(lm.state_dict(), ckpt_dir / "model.pth")
+    rm = load_reward_model(ckpt_dir / "model.pth", "cpu", torch.bfloat16)
+    assert isinstance(rm, RewardModel) and rm.backbone_model is rm.backbone and not rm.training
+    head = rm.backbone.output
+    assert tuple(head.weight.shape) == (2, lm.config.dim) and head.out_features == 2
+    assert head.weight.dtype == torch.bfloat16 and not head.weight.requires_grad and int(head.weight.count_nonzero()) == 0
+    assert torch.equal(rm.backbone.layers[1].feed_forward.w2.weight, lm.layers[1].feed_forward.w2.weight)
+    for bad in ("model_int8.pth", "model_int4.g128.pth"):
+        (ckpt_dir / bad).write_bytes(b"")
+        with pytest.raises(NotImplementedError):
+            load_reward_model(ckpt_dir / bad, "cpu")
+    with pytest.raises(FileNotFoundError):
+        load_reward_model(ckpt_dir / "absent.pth", "cpu")
+    with pytest.raises(NotImplementedError):
+        load_reward_model(ckpt_dir / "model.pth", "cpu", use_tp=True)
+
+    big = nn.Module()
+    big.output = nn.Linear(8, 30000, bias=False)
+    w = big.output.weight.detach().clone()
+    apply_reward_modeling_head(big, init_scheme="semantic")
+    assert torch.equal(big.output.weight[0], w[29906]) and torch.equal(big.output.weight[1], -w[29896])
+    apply_reward_modeling_head(big, init_scheme="random")
+    first = big.output.weight.detach().clone()
+    apply_reward_modeling_head(big, init_scheme="random")
+    assert tuple(first.shape) == (2, 8) and torch.equal(first, big.output.weight) and float(first.abs().max()) > 0
+    with pytest.raises(ValueError):
+        apply_reward_modeling_head(big, init_scheme="other")

@@ -7,7 +7,7 @@ import torch
 
 import easy_to_hard_amd as e2h
 from easy_to_hard_amd import ops
-from easy_to_hard_amd.generate import GraphedDecodeStep, decode_one_token, generate, load_model, prefill
+from easy_to_hard_amd.generate import GraphedDecodeStep, decode_one_token, generate, load_model, load_reward_model, model_score, prefill
 from easy_to_hard_amd.model import Transformer, init_random_
 from tests.helpers import randn_bf16
 
@@ -155,3 +155,33 @@ def test_loader_rejects_what_it_cannot_interpret(tmp_path):
         load_model(ckpt_dir / "missing_int8.pth", DEV)
     with pytest.raises(NotImplementedError):
         load_model(wrong, DEV, use_tp=True)
+
+
+def test_reward_model_loader_with_on_the_fly_int8(tmp_path):
+    """load_reward_model(..., on_the_fly_8bit_quantization=True) = the reference's _load_reward_model followed by the
+    quantization step of its main (inference_reward.py:94-118, :171-178): every linear, the two-row head included, becomes
+    a WeightOnlyInt8Linear on the GPU; scores stay within the weights' int8 quantization error (about 1 / 127.5 of each row's
+    largest weight per weight, through two layers) of the unquantized bfloat16 model's -- arithmetic parity of the int8
+    scoring pass against its oracle twin is tests/test_gpu_model.py::test_int8_on_the_fly_reward_scoring."""
+    ckpt_dir = tmp_path / "tiny-test"
+    ckpt_dir.mkdir()
+    lm = Transformer.from_name("tiny-test")
+    init_random_(lm, seed=11, std=0.05)
+    torch.save(lm.state_dict(), ckpt_dir / "model.pth")
+    plain = load_reward_model(ckpt_dir / "model.pth", DEV, torch.bfloat16)
+    head = randn_bf16((2, lm.config.dim), std=0.05, seed=12).to(DEV)
+    plain.backbone.output.weight.data.copy_(head)
+    quant = load_reward_model(ckpt_dir / "model.pth", DEV, torch.bfloat16)
+    quant.backbone.output.weight.data.copy_(head)
+    quant = e2h.WeightOnlyInt8QuantHandler(quant).convert_for_runtime_on_the_fly().eval()
+    direct = load_reward_model(ckpt_dir / "model.pth", DEV, torch.bfloat16, on_the_fly_8bit_quantization=True)
+    for mod in (quant, direct):
+        assert isinstance(mod.backbone.output, e2h.WeightOnlyInt8Linear) and mod.backbone.output.out_features == 2
+        assert isinstance(mod.backbone.layers[0].attention.wqkv, e2h.WeightOnlyInt8Linear)
+        assert mod.backbone.layers[0].attention.wqkv.weight.is_cuda
+    ids = torch.randint(0, lm.config.vocab_size, (3, 24), generator=torch.Generator().manual_seed(2)).to(DEV)
+    assert int(model_score(direct, ids).count_nonzero()) == 0          # zero head, as loaded
+    want, got = model_score(plain, ids).float(), model_score(quant, ids).float()
+    assert got.shape == (3, 24)
+    assert float((got - want).abs().max()) <= 1e-1 * float(want.abs().max())
+    assert torch.equal(model_score(direct, ids), torch.zeros_like(got, dtype=torch.bfloat16))
