@@ -98,6 +98,11 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.int8_gemm_wave_cols = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "int4_gemm_tile")) {
+    if (value != 0 && value != 128 && value != 256) return E2H_ERR_BAD_OPTION;
+    o.int4_gemm_tile = value;
+    return E2H_OK;
+  }
   if (!strcmp(name, "int8_gemm_tile")) {
     if (value != 0 && value != 128 && value != 256) return E2H_ERR_BAD_OPTION;
     o.int8_gemm_tile = value;

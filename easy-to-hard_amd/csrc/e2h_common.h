@@ -50,6 +50,7 @@ struct Options {
   int attention_waves;     // 0 = by cache length, else 4 or 8 waves per decode-attention workgroup
   int attention_no_mfma;   // 1 = grouped-query decode attention stays on the float32 vector kernel
   int int8_gemm_tile;      // 0 = heuristic, else 128 or 256 rows per workgroup in the many-row int8 matmul
+  int int4_gemm_tile;      // 0 = heuristic, else 128 or 256 rows per workgroup in the many-row int4 matmul
   int int8_gemm_waves;     // 0 or 4 = the 256-row workgroup is the four-wave kernel, 8 = the eight-wave one
   int int8_gemm_wave_cols; // four-wave kernel: 0 or 4 = every wave 256 rows x 64 columns, 2 = 128 rows x 128 columns
 };

@@ -747,6 +747,21 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
     a.y = y + m0 * a.N;
     a.M = static_cast<int>(m_total - m0 < max_rows ? m_total - m0 : max_rows);
     a.xsum = nullptr;
+    if (mt == 4 && wide_ok && !options().int4_no_gemm32) {
+      // 256 x 256 outputs per workgroup (dequantize-to-bfloat16 kernel, no group sums of x): a 256-row workgroup takes
+      // about 1.8 x as long as a 128-row one of the 32x32-tile kernel below, so it wins when it needs fewer than 1 / 1.8
+      // as many rounds of workgroups over the chip's CUs
+      const long long wgs256 = static_cast<long long>((a.M + 255) / 256) * ((a.N + 255) / 256);
+      const long long wgs128 = static_cast<long long>((a.M + 127) / 128) * ((a.N + 255) / 256);
+      const long long rounds256 = (wgs256 + kCUs - 1) / kCUs, rounds128 = (wgs128 + kCUs - 1) / kCUs;
+      const bool enough = options().int4_gemm32_min_rows > 0 ? a.M >= options().int4_gemm32_min_rows : wgs128 >= 320;
+      const bool big = options().int4_gemm_tile ? options().int4_gemm_tile == 256 : (enough && rounds256 * 20 <= rounds128 * 11);
+      if (big && a.K % 256 == 0) {
+        const int rc128 = int4_gemm128(a.x, a.packed, a.sz, a.y, a.M, a.N, a.K, groupsize, a.stream);
+        if (rc128 != E2H_OK) return rc128;
+        continue;
+      }
+    }
     if (mt == 4 && wide_ok && (sh.t == 1 || sh.t == 2) && workspace && !options().int4_no_xsum) {
       // many rows: one pass over x leaves its group sums in the workspace's partial-tile area (unused here: no K split)
       const int stride = ((a.M + 63) / 64) * 64;

@@ -93,5 +93,10 @@ int launch_x_group_sums(const uint16_t *x, float *out, int M, int K, int stride,
 int int4_gemm32(const uint16_t *x, const int32_t *packed, const uint16_t *sz, uint16_t *y, const float *xsum, int xsum_stride,
                 int M, int N, int K, int groupsize, hipStream_t stream);
 
+// Many-row int4 matmul, 256 x 256 outputs per workgroup, weights dequantized to bfloat16 on the way into the matrix
+// cores (e2h_int4_gemm128.hip); needs no scratch memory.
+int int4_gemm128(const uint16_t *x, const int32_t *packed, const uint16_t *sz, uint16_t *y, int M, int N, int K, int groupsize,
+                 hipStream_t stream);
+
 }  // namespace e2h
 #endif

@@ -463,6 +463,54 @@ def test_int8_many_rows_at_the_reward_scoring_size():
     y_int = qo.int8_linear_reference_rounding(bf16_to_np(x[-3:]), q, s)
     assert np.array_equal(bf16_to_np(y[-3:].cpu()), y_int)
 
+@pytest.mark.parametrize("g", [32, 64, 128])
+@pytest.mark.parametrize("m,n,k", [(300, 264, 512), (1000, 520, 256), (257, 136, 768), (257, 136, 384), (512, 4096, 4096)])
+def test_int4_gemm128_dequantizing_kernel_matches_oracle_and_32x32_tile_kernel(m, n, k, g):
+    """The 256 x 256-output kernel (weights dequantized to bfloat16 on the way into the matrix cores, the reference
+    kernel's arithmetic) against the oracle and against the 128-row kernel (exact products, scale applied in float32):
+    ragged M and N, one and several trips of its two-block loop, every group size; K = 384 is not a multiple of 256 and
+    stays on the 128-row kernel.  The two kernels differ by the bfloat16 rounding of each weight (2^-9 relative, random
+    sign) on top of the output rounding."""
+    if k == 4096 and g != 128:
+        pytest.skip("large shape: one group size only")
+    codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=m + n + g)
+    x = randn_bf16((m, k), std=1.0, seed=m + 2)
+    _lib.set_option("int4_gemm32_min_rows", 65)
+    try:
+        _lib.set_option("int4_gemm_tile", 256)
+        y, _ = _check_int4(x, codes, sz, packed_d, sz_d, g)
+        _lib.set_option("int4_gemm_tile", 128)
+        y2, _ = _check_int4(x, codes, sz, packed_d, sz_d, g)
+    finally:
+        _lib.set_option("int4_gemm_tile", 0)
+        _lib.set_option("int4_gemm32_min_rows", 0)
+    bound = 2.0 ** -6 * y2.float().abs().max().item()
+    assert (y.float() - y2.float()).abs().max().item() <= bound
+    if k % 256:
+        assert torch.equal(y, y2)
+
+
+def test_int4_gemm128_with_weights_that_dequantize_exactly():
+    """Scales that are powers of two and zeros that are small multiples of them make every s * (q - 8) + z a bfloat16
+    value, and x in {-1, 0, 1} makes every product and partial sum exact: the dequantizing kernel must then return
+    bfloat16(exact sum) for every element, whatever the order of its additions."""
+    m, n, k, g = 300, 264, 512, 64
+    gen = torch.Generator().manual_seed(21)
+    codes = torch.randint(0, 16, (n, k), generator=gen, dtype=torch.int32)
+    scales = torch.pow(2.0, torch.randint(-6, -2, (k // g, n), generator=gen).float())
+    zeros = scales * torch.randint(-8, 9, (k // g, n), generator=gen).float()
+    sz = torch.stack([scales, zeros], dim=-1).to(torch.bfloat16)
+    x = torch.randint(-1, 2, (m, k), generator=gen).to(torch.bfloat16)
+    w = (codes.float() - 8) * scales.t().repeat_interleave(g, 1) + zeros.t().repeat_interleave(g, 1)
+    want = (x.double() @ w.double().t()).to(torch.bfloat16)
+    packed_d = ops.int4_pack(codes.to(DEV), 8)
+    _lib.set_option("int4_gemm_tile", 256)
+    try:
+        got = ops.int4_mm_direct(x.to(DEV), packed_d, g, sz.to(DEV))
+    finally:
+        _lib.set_option("int4_gemm_tile", 0)
+    assert torch.equal(got.cpu(), want)
+
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["int8", "int4"])
@@ -488,15 +536,19 @@ def test_many_row_kernels_with_an_output_that_is_only_2_byte_aligned(mode):
                 assert buf[0].item() == 0 and buf[1 + m * n:].abs().max().item() == 0
         else:
             codes, sz, packed_d, sz_d = _int4_case(n, k, g, 8, seed=12)
-            y_ref = ops.int4_mm_direct(x, packed_d, g, sz_d)
-            rc = lib.e2h_int4_mm(ops._ptr(x), ops._ptr(packed_d), ops._ptr(sz_d), ctypes.c_void_p(buf.data_ptr() + 2), m, n, k, g, 8, ops._ptr(ws), ws.numel(),
-                                 ops._stream(x))
-            _lib.check(rc, "e2h_int4_mm")
-            assert torch.equal(buf[1:1 + m * n].view(m, n), y_ref)
-            assert buf[0].item() == 0 and buf[1 + m * n:].abs().max().item() == 0
+            for tile in (128, 256):
+                _lib.set_option("int4_gemm_tile", tile)
+                buf.zero_()
+                y_ref = ops.int4_mm_direct(x, packed_d, g, sz_d)
+                rc = lib.e2h_int4_mm(ops._ptr(x), ops._ptr(packed_d), ops._ptr(sz_d), ctypes.c_void_p(buf.data_ptr() + 2), m, n, k, g, 8, ops._ptr(ws),
+                                     ws.numel(), ops._stream(x))
+                _lib.check(rc, "e2h_int4_mm")
+                assert torch.equal(buf[1:1 + m * n].view(m, n), y_ref)
+                assert buf[0].item() == 0 and buf[1 + m * n:].abs().max().item() == 0
     finally:
         _lib.set_option("int4_gemm32_min_rows", 0)
         _lib.set_option("int8_gemm_tile", 0)
+        _lib.set_option("int4_gemm_tile", 0)
 
 
 @pytest.mark.gpu
