@@ -734,7 +734,18 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
   int64_t max_rows = rows_by_bytes < rows_by_grid ? rows_by_bytes : rows_by_grid;
   max_rows -= max_rows % (16 * mt);
   if (max_rows < 16 * mt) return E2H_ERR_BAD_SHAPE;
-  if (mt == 4 && wide_ok && workspace && !options().int4_no_xsum) {
+  // 256 x 256 outputs per workgroup (dequantize-to-bfloat16 kernel, no group sums of x) or 128 x 256 (32x32-tile kernel
+  // with group sums from a pre-pass): a 256-row workgroup takes about 1.8 x as long as a 128-row one, so it wins when it
+  // needs fewer than 1 / 1.8 as many rounds of workgroups over the chip's CUs
+  const auto takes_256_row_kernel = [&](int64_t rows) {
+    if (!(mt == 4 && wide_ok && !options().int4_no_gemm32 && a.K % 256 == 0)) return false;
+    const long long wgs256 = static_cast<long long>((rows + 255) / 256) * ((a.N + 255) / 256);
+    const long long wgs128 = static_cast<long long>((rows + 127) / 128) * ((a.N + 255) / 256);
+    const long long rounds256 = (wgs256 + kCUs - 1) / kCUs, rounds128 = (wgs128 + kCUs - 1) / kCUs;
+    const bool enough = options().int4_gemm32_min_rows > 0 ? rows >= options().int4_gemm32_min_rows : wgs128 >= 320;
+    return options().int4_gemm_tile ? options().int4_gemm_tile == 256 : (enough && rounds256 * 20 <= rounds128 * 11);
+  };
+  if (mt == 4 && wide_ok && workspace && !options().int4_no_xsum && !takes_256_row_kernel(a.M)) {
     // many rows: the pre-pass keeps (K / g) sums per row in the workspace; slice M so that they fit rather than fall
     // back to the kernels that form the sums themselves (K = 22016 at g = 64: 24k rows per slice with 32 MB)
     const int64_t avail = workspace_bytes - static_cast<int64_t>(kTicketBytes);
@@ -747,20 +758,10 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
     a.y = y + m0 * a.N;
     a.M = static_cast<int>(m_total - m0 < max_rows ? m_total - m0 : max_rows);
     a.xsum = nullptr;
-    if (mt == 4 && wide_ok && !options().int4_no_gemm32) {
-      // 256 x 256 outputs per workgroup (dequantize-to-bfloat16 kernel, no group sums of x): a 256-row workgroup takes
-      // about 1.8 x as long as a 128-row one of the 32x32-tile kernel below, so it wins when it needs fewer than 1 / 1.8
-      // as many rounds of workgroups over the chip's CUs
-      const long long wgs256 = static_cast<long long>((a.M + 255) / 256) * ((a.N + 255) / 256);
-      const long long wgs128 = static_cast<long long>((a.M + 127) / 128) * ((a.N + 255) / 256);
-      const long long rounds256 = (wgs256 + kCUs - 1) / kCUs, rounds128 = (wgs128 + kCUs - 1) / kCUs;
-      const bool enough = options().int4_gemm32_min_rows > 0 ? a.M >= options().int4_gemm32_min_rows : wgs128 >= 320;
-      const bool big = options().int4_gemm_tile ? options().int4_gemm_tile == 256 : (enough && rounds256 * 20 <= rounds128 * 11);
-      if (big && a.K % 256 == 0) {
-        const int rc128 = int4_gemm128(a.x, a.packed, a.sz, a.y, a.M, a.N, a.K, groupsize, a.stream);
-        if (rc128 != E2H_OK) return rc128;
-        continue;
-      }
+    if (takes_256_row_kernel(a.M)) {
+      const int rc128 = int4_gemm128(a.x, a.packed, a.sz, a.y, a.M, a.N, a.K, groupsize, a.stream);
+      if (rc128 != E2H_OK) return rc128;
+      continue;
     }
     if (mt == 4 && wide_ok && (sh.t == 1 || sh.t == 2) && workspace && !options().int4_no_xsum) {
       // many rows: one pass over x leaves its group sums in the workspace's partial-tile area (unused here: no K split)

@@ -242,6 +242,27 @@ def test_34b_linear_shapes_g64(n, k, m):
     assert qo.elementwise_violations(got, y_ref) == 0.0
 
 
+def test_34b_prefill_rows_8192x22016_g64_in_one_launch():
+    """The prefill of the 34B configuration gives every linear 64 x 512 = 32768 rows; with K = 22016 at group size 64 the
+    group sums of x for that many rows do not fit the workspace, and a call that needs them is cut into slices of rows.
+    The 256-row kernel needs none: the whole call must go to it in one piece (sampled rows and columns against the
+    oracle; rows on both sides of where the slices would have been cut)."""
+    n, k, g, m = 8192, 22016, 64, 32768
+    packed, sz = _big_int4_weight(n, k, g, seed=77)
+    gen = torch.Generator(device=DEV).manual_seed(78)
+    x = torch.randn((m, k), generator=gen, device=DEV).to(torch.bfloat16)
+    y = ops.int4_mm_direct(x, packed, g, sz)
+    rows = torch.tensor([0, 1, 255, 256, 12345, 24319, 24320, 24321, 32000, 32767], device=DEV)
+    tiles, cols = _sampled_columns(n, 29, seed=3)
+    y_ref = _oracle_columns(x[rows].cpu(), packed, sz, tiles, cols, g)
+    got = bf16_to_np(y[rows][:, cols])
+    assert qo.normwise_rel_err(got, y_ref) <= TOL
+    assert qo.elementwise_violations(got, y_ref) == 0.0
+    # the same rows as a small call (the exact-product kernel): agreement to the bfloat16 rounding of the weights
+    small = ops.int4_mm_direct(x[rows].contiguous(), packed, g, sz)
+    assert (small.float() - y[rows].float()).abs().max().item() <= 2.0 ** -6 * small.float().abs().max().item()
+
+
 @pytest.mark.parametrize("m", [64, 32])
 def test_34b_gated_pair_2x22016x8192_g64(m):
     n, k, g = 22016, 8192, 64
