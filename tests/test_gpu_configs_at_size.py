@@ -152,19 +152,17 @@ def test_output_head_32000x4096_g128(m):
     assert qo.elementwise_violations(got, y_ref) == 0.0
 
 
-def test_7b_int4_g128_batch32_decode_against_the_oracle_model():
-    """Random-init Llama-2-7B-shaped model, int4 g128, batch 32, prompt of 256 uniform token ids, seed 1234: prefill, then
-    decode steps through the fused kernels, every step compared with a float32 oracle twin that sees the same tokens
-    (teacher forcing).  Thirty-two layers of bfloat16 activations amplify rounding differences, so the gate on the logits
-    is the larger of 2e-2 (normwise) and 1.5 x the distance of the reference's own arithmetic (bfloat16 dequantized
-    weights, torch's bfloat16 F.linear) from the same oracle; the greedy tokens must agree with the oracle's at least as
-    often as that arithmetic's do (less 5 %).  Finally the HIP-graph replayed step must reproduce the
-    eager step bit for bit at this size."""
+def _decode_against_the_oracle_model(cfg, g, bsz, t_prompt, steps, label):
+    """Random-init model of shape `cfg`, int4 with group size g, batch bsz, prompt of t_prompt uniform token ids, seed
+    1234: prefill, then decode steps through the fused kernels, every step compared with a float32 oracle twin that sees
+    the same tokens (teacher forcing).  Many layers of bfloat16 activations amplify rounding differences, so the gate on
+    the logits is the larger of 2e-2 (normwise) and 1.5 x the distance of the reference's own arithmetic (bfloat16
+    dequantized weights, torch's bfloat16 F.linear) from the same oracle; the greedy tokens must agree with the oracle's at
+    least as often as that arithmetic's do (less 5 %).  Finally the HIP-graph replayed step must reproduce the eager step
+    bit for bit at this size."""
     from easy_to_hard_amd.generate import GraphedDecodeStep
 
-    cfg = ModelArgs.from_name("7B")
-    bsz, t_prompt, steps = 32, 256, 8
-    model = random_quantized_transformer(cfg, "int4", 128, device=DEV, seed=1234)
+    model = random_quantized_transformer(cfg, "int4", g, device=DEV, seed=1234)
     model.setup_caches(bsz, t_prompt + steps + 8)
     oracle = _oracle_twin(model, torch.float32)
     ref_arith = _oracle_twin(model, torch.bfloat16)
@@ -190,7 +188,7 @@ def test_7b_int4_g128_batch32_decode_against_the_oracle_model():
             d, e = compare(lq, ref_arith(cur, step_pos), oracle(cur, step_pos), f"decode step {i}")
             same_ref, same = same_ref + d, same + e
             cur = lq[:, -1].float().argmax(-1, keepdim=True)
-        print("7B int4 g128 bs32: (step, normwise logit error vs float32 oracle, same for the reference's bf16 arithmetic):", report)
+        print(f"{label}: (step, normwise logit error vs float32 oracle, same for the reference's bf16 arithmetic):", report)
         total = (steps + 1) * bsz
         print(f"greedy tokens equal to the float32 oracle's: {same} of {total}; the reference's bf16 arithmetic: {same_ref} of {total}")
         # random-init logits are near ties (vocabulary of 32000, logit spread ~1.3): rounding noise flips some arg-maxes in
@@ -207,6 +205,21 @@ def test_7b_int4_g128_batch32_decode_against_the_oracle_model():
             blk.attention.kv_cache.v_cache[:, :, 0] = v0
         replay = stepper.step(cur, step_pos).clone()
         assert torch.equal(eager, replay)
+
+
+def test_7b_int4_g128_batch32_decode_against_the_oracle_model():
+    """The 7B decode configuration at its full size: 32 layers, batch 32, prompt 256."""
+    _decode_against_the_oracle_model(ModelArgs.from_name("7B"), 128, 32, 256, 8, "7B int4 g128 bs32")
+
+
+def test_34b_int4_g64_batch64_decode_against_the_oracle_model():
+    """The 34B decode configuration (dim 8192, 64 query / 8 kv heads, FFN 22016, group size 64, batch 64, prompt 512) at
+    full width with the first 8 of its 48 layers: every kernel of the step runs at its real shape (32768-row prefill
+    matmuls, two-slab 64-row decode launches, grouped-query attention on the matrix cores), and the float32 oracle twin
+    of 8 layers fits next to it."""
+    cfg = ModelArgs.from_name("34B")
+    cfg.n_layer = 8
+    _decode_against_the_oracle_model(cfg, 64, 64, 512, 4, "34B (8 layers) int4 g64 bs64")
 
 
 # ---- the 34B int4 g64 decode configuration: every linear shape at 64 rows ----------------------------------------
