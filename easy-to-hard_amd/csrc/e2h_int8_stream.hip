@@ -286,20 +286,30 @@ __global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint
     if (tid == 0) __hip_atomic_store(ws_ticket + wg_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (kg == 0) {
       const float *all = ws_partial + wg_tile * S * tile_floats + static_cast<size_t>(wave_n) * kSlots * 64 + lane;
-      for (int s2 = 0; s2 < S; ++s2) {
-        float v[kSlots];
+      // the loads of four slices are issued before the first addition (one round trip to the memory side instead of
+      // one per slice); the additions keep the slice order
+      for (int s0 = 0; s0 < S; s0 += 4) {
+        float v[4][kSlots];
 #pragma unroll
-        for (int slot = 0; slot < kSlots; ++slot)
-          v[slot] = __hip_atomic_load(all + s2 * tile_floats + slot * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int u = 0; u < 4; ++u) {
+          const int s2 = s0 + u < S ? s0 + u : S - 1;  // past the end: a slice read again and not added
 #pragma unroll
-        for (int t = 0; t < T; ++t)
+          for (int slot = 0; slot < kSlots; ++slot)
+            v[u][slot] = __hip_atomic_load(all + s2 * tile_floats + slot * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
+        for (int u = 0; u < 4; ++u) {
+          if (s0 + u >= S) break;  // uniform
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int slot = (t * MT + mt) * 4 + r;
-              acc[t][mt][r] = s2 == 0 ? v[slot] : acc[t][mt][r] + v[slot];
-            }
+          for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int slot = (t * MT + mt) * 4 + r;
+                acc[t][mt][r] = s0 + u == 0 ? v[u][slot] : acc[t][mt][r] + v[u][slot];
+              }
+        }
       }
     }
   }
