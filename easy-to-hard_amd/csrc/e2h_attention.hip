@@ -360,12 +360,45 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
 // round trip for the whole row up to BLOCK * 8 * kPieces values); longer rows re-read the rest.
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ delta,
+                                                        const float *__restrict__ psum, int slices,
                                                         const uint16_t *__restrict__ w, uint16_t *__restrict__ h_out,
                                                         uint16_t *__restrict__ y, int dim, float eps) {
   constexpr int kPieces = 2, kStride = BLOCK * 8, kWaves = BLOCK / 64;
+  constexpr int kMaxSlices = 4;  // slices whose loads are all issued before the first addition
   const size_t row = blockIdx.x;
   const uint16_t *xr = x + row * dim;
   const uint16_t *dr_row = delta ? delta + row * dim : nullptr;
+  // psum: the term to add arrives as float32 partial sums [slices][rows][dim] of a matmul split along K; the term is
+  // bf16(p[0] + p[1] + .. in slice order), the value the matmul's own combine step would have stored
+  const size_t slice_floats = static_cast<size_t>(gridDim.x) * dim;
+  const float *pr = psum ? psum + row * dim : nullptr;
+  auto sum_slices = [&](int i) {
+    f32x4_t lo[kMaxSlices], hi[kMaxSlices];
+#pragma unroll
+    for (int u = 0; u < kMaxSlices; ++u) {
+      const int s2 = u < slices ? u : slices - 1;
+      lo[u] = *reinterpret_cast<const f32x4_t *>(pr + s2 * slice_floats + i);
+      hi[u] = *reinterpret_cast<const f32x4_t *>(pr + s2 * slice_floats + i + 4);
+    }
+    f32x4_t a = lo[0], b = hi[0];
+#pragma unroll
+    for (int u = 1; u < kMaxSlices; ++u)
+      if (u < slices) {
+        a += lo[u];
+        b += hi[u];
+      }
+    for (int s2 = kMaxSlices; s2 < slices; ++s2) {
+      a += *reinterpret_cast<const f32x4_t *>(pr + s2 * slice_floats + i);
+      b += *reinterpret_cast<const f32x4_t *>(pr + s2 * slice_floats + i + 4);
+    }
+    u32x4_t d;
+    d[0] = static_cast<uint32_t>(f32_to_bf16_rne(a[0])) | (static_cast<uint32_t>(f32_to_bf16_rne(a[1])) << 16);
+    d[1] = static_cast<uint32_t>(f32_to_bf16_rne(a[2])) | (static_cast<uint32_t>(f32_to_bf16_rne(a[3])) << 16);
+    d[2] = static_cast<uint32_t>(f32_to_bf16_rne(b[0])) | (static_cast<uint32_t>(f32_to_bf16_rne(b[1])) << 16);
+    d[3] = static_cast<uint32_t>(f32_to_bf16_rne(b[2])) | (static_cast<uint32_t>(f32_to_bf16_rne(b[3])) << 16);
+    return d;
+  };
+  const bool adds = delta || psum;
   auto add_round = [](u32x4_t a, u32x4_t d) {  // bf16(x + delta), value by value
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -402,6 +435,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
     if (i < dim) {
       keep[p] = *reinterpret_cast<const u32x4_t *>(xr + i);
       if (delta) keepd[p] = *reinterpret_cast<const u32x4_t *>(dr_row + i);
+      else if (psum) keepd[p] = sum_slices(i);
       keepw[p] = *reinterpret_cast<const u32x4_t *>(w + i);  // needed only after the reduction
     }
   }
@@ -410,7 +444,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
   for (int p = 0; p < kPieces; ++p) {
     const int i = threadIdx.x * 8 + p * kStride;
     if (i < dim) {
-      if (delta) {
+      if (adds) {
         keep[p] = add_round(keep[p], keepd[p]);
         *reinterpret_cast<u32x4_t *>(h_out + row * dim + i) = keep[p];
       }
@@ -419,8 +453,8 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
   }
   for (int i = threadIdx.x * 8 + kPieces * kStride; i < dim; i += kStride) {
     u32x4_t raw = *reinterpret_cast<const u32x4_t *>(xr + i);
-    if (delta) {
-      raw = add_round(raw, *reinterpret_cast<const u32x4_t *>(dr_row + i));
+    if (adds) {
+      raw = add_round(raw, delta ? *reinterpret_cast<const u32x4_t *>(dr_row + i) : sum_slices(i));
       *reinterpret_cast<u32x4_t *>(h_out + row * dim + i) = raw;
     }
     ss = sum_sq(raw, ss);
@@ -433,7 +467,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
 #pragma unroll
   for (int wv = 0; wv < kWaves; ++wv) ss += part[wv];
   const float inv = rsqrtf(ss / static_cast<float>(dim) + eps);
-  const uint16_t *src = delta ? h_out + row * dim : xr;
+  const uint16_t *src = adds ? h_out + row * dim : xr;
   uint16_t *yr = y + row * dim;
 #pragma unroll
   for (int p = 0; p < kPieces; ++p) {
@@ -515,12 +549,14 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
 }
 
 // few rows (decode): 512 threads so that a 4096-wide row is one piece per thread; many rows: 256-thread workgroups
-void launch_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *w, uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim,
-                    float eps, hipStream_t stream) {
+void launch_rmsnorm(const uint16_t *x, const uint16_t *delta, const float *psum, int slices, const uint16_t *w, uint16_t *h_out, uint16_t *y,
+                    int64_t rows, int64_t dim, float eps, hipStream_t stream) {
   if (rows <= 512 && dim >= 4096)
-    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(static_cast<unsigned>(rows)), dim3(512), 0, stream, x, delta, w, h_out, y, static_cast<int>(dim), eps);
+    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(static_cast<unsigned>(rows)), dim3(512), 0, stream, x, delta, psum, slices, w, h_out, y,
+                       static_cast<int>(dim), eps);
   else
-    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, x, delta, w, h_out, y, static_cast<int>(dim), eps);
+    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, x, delta, psum, slices, w, h_out, y,
+                       static_cast<int>(dim), eps);
 }
 
 template <int D, int NW>
@@ -581,7 +617,7 @@ extern "C" int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *
   if (!x || !weight || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, nullptr, weight, nullptr, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, nullptr, nullptr, 0, weight, nullptr, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 
@@ -590,7 +626,16 @@ extern "C" int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const u
   if (!x || !delta || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(delta) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, delta, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, delta, nullptr, 0, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  return launch_status();
+}
+
+extern "C" int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *weight, uint16_t *h_out,
+                                        uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream) {
+  if (!x || !partials || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
+  if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX || slices < 1 || slices > 64) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(partials) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
+  launch_rmsnorm(x, nullptr, partials, slices, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 

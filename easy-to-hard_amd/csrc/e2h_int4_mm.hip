@@ -101,7 +101,11 @@ struct Tuning {
 // epilogue rounds it to bfloat16, rotates the interleaved pairs of the q and k heads in float32 by the angle of
 // position input_pos[0] (reference models/model.py:400-412), and writes q to q_out [B, H, D] and k, v straight
 // into the caches [B, Hkv, S, D] at that position (KVCache.update, reference models/model.py:94-104).
-enum Epilogue { kPlain = 0, kGate = 1, kRope = 2 };
+//
+// PARTIAL: the workgroup's float32 sums over its K slice go to slice blockIdx.y of a row-major [S][M][N] array and the
+// launch ends there: no tickets, no meeting of the slices.  The consumer (the residual add + RMSNorm that follows the
+// wo and w2 projections of a decoder block, reference models/model.py:279-282) adds the slices in slice order.
+enum Epilogue { kPlain = 0, kGate = 1, kRope = 2, kPartial = 3 };
 
 struct RopeArgs {
   const uint16_t *freqs;     // [>= S, D/2, 2] bf16 (cos, sin)
@@ -426,6 +430,23 @@ __global__ __launch_bounds__(64 * WN * WK) void int4_skinny_mm_kernel(
     }
   }
 
+  if constexpr (EPI == kPartial) {
+    if (kg != 0) return;
+    float *out = ws_partial + static_cast<size_t>(ks) * M * N;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const int n = 16 * (tile16_0 + t) + c;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int m = m_base + 16 * mt + 4 * b + q;
+          if (n < N && m < M) out[static_cast<size_t>(m) * N + n] = acc[t][mt][q];
+        }
+    }
+    return;
+  }
+
   // ---- epilogue 2: combine the K slices of different workgroups ------------------------------------
   // Partial tiles and the ticket travel as device-scope relaxed atomics (written through to, and read from,
   // the memory side, so no cache write-back or invalidate is needed); the stores are complete before the
@@ -638,6 +659,14 @@ int dispatch_ikt(int ikt, int mt, Shape sh, const LaunchArgs &a) {
 constexpr size_t kTicketBytes = 64 * 1024;  // 16384 tickets
 constexpr int kCUs = 256;
 
+// K slices for the 32-row decode shape (4 column waves x 2 k-groups): narrow matrices split K over S workgroups as long
+// as that does not exceed one workgroup per CU and leaves every k-group at least four chunks
+inline int decode_k_slices(int blocks, int nchunks) {
+  int s = 1;
+  while (s < 4 && blocks * s * 2 <= kCUs && nchunks / (2 * s * 2) >= 4) s *= 2;
+  return s;
+}
+
 }  // namespace
 }  // namespace e2h
 
@@ -701,8 +730,7 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
   if (wide_ok && mt <= 2) {
     sh = Shape{1, 4, 2};
     const int blocks = ((tiles16 + 3) / 4) * m_chunks;
-    if (have_ws)
-      while (s < 4 && blocks * s * 2 <= kCUs && nchunks / (2 * s * sh.wk) >= 4) s *= 2;
+    if (have_ws) s = decode_k_slices(blocks, nchunks);
     // More column blocks than CUs: a wave with two column tiles takes about 1.5x as long as with one, and halving the
     // number of workgroups saves more than that whenever one tile per wave needs a second round of workgroups
     // (measured: 10240 x 8192 at 64 rows 32.9 instead of 44.5 us, 32000 x 8192 71.5 instead of 97.7,
@@ -944,5 +972,55 @@ extern "C" int e2h_int4_mm_rope_kv(const uint16_t *x, const int32_t *packed, con
     case 32: return wide ? launch<32, 8, 2, 2, 4, 2, kRope>(a) : two ? launch<32, 8, 2, 1, 4, 2, kRope>(a) : launch<32, 8, 1, 1, 4, 2, kRope>(a);
     case 64: return wide ? launch<64, 8, 2, 2, 4, 2, kRope>(a) : two ? launch<64, 8, 2, 1, 4, 2, kRope>(a) : launch<64, 8, 1, 1, 4, 2, kRope>(a);
     default: return wide ? launch<128, 8, 2, 2, 4, 2, kRope>(a) : two ? launch<128, 8, 2, 1, 4, 2, kRope>(a) : launch<128, 8, 1, 1, 4, 2, kRope>(a);
+  }
+}
+
+namespace e2h {
+namespace {
+
+// shape checks shared by the two entry points below; returns the number of K slices (>= 1) or a negative status
+int partial_slices_for(int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles) {
+  if (groupsize != 32 && groupsize != 64 && groupsize != 128) return E2H_ERR_BAD_GROUPSIZE;
+  if (inner_k_tiles != 8) return E2H_ERR_BAD_INNER_K_TILES;
+  if (m < 1 || m > 64 || n < 8 || k < 1 || (n % 8) != 0 || n > INT32_MAX || k > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if (k % groupsize != 0) return E2H_ERR_BAD_GROUPSIZE;
+  if (k % 128 != 0) return E2H_ERR_BAD_INNER_K_TILES;
+  if (n * k / 2 >= (int64_t{1} << 32) || (k / groupsize) * n * 4 >= (int64_t{1} << 32)) return E2H_ERR_BAD_SHAPE;
+  const int mt = m <= 16 ? 1 : 2;
+  const int m_chunks = static_cast<int>((m + 16 * mt - 1) / (16 * mt));
+  const int tiles16 = static_cast<int>((n + 15) / 16);
+  const int nchunks = static_cast<int>(k / 128);
+  int s = decode_k_slices(((tiles16 + 3) / 4) * m_chunks, nchunks);
+  if (options().int4_k_slices > 0) s = options().int4_k_slices;
+  if (s > nchunks) s = nchunks;
+  return s;
+}
+
+}  // namespace
+}  // namespace e2h
+
+extern "C" int e2h_int4_mm_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles) {
+  return e2h::partial_slices_for(m, n, k, groupsize, inner_k_tiles);
+}
+
+extern "C" int e2h_int4_mm_partials(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, float *partials,
+                                    int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, int slices, void *stream) {
+  using namespace e2h;
+  if (!x || !packed || !scales_and_zeros || !partials) return E2H_ERR_NULL_POINTER;
+  const int want = partial_slices_for(m, n, k, groupsize, inner_k_tiles);
+  if (want < 0) return want;
+  if (slices != want) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(packed) || !aligned16(scales_and_zeros) || (reinterpret_cast<uintptr_t>(partials) & 3u)) return E2H_ERR_MISALIGNED;
+  LaunchArgs a;
+  a.x = x; a.packed = packed; a.sz = scales_and_zeros; a.packed2 = nullptr; a.sz2 = nullptr; a.y = nullptr;
+  a.rope = RopeArgs{}; a.xsum = nullptr; a.xsum_stride = 0;
+  a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k);
+  a.S = slices; a.ws_partial = partials; a.ws_ticket = nullptr;
+  a.stream = static_cast<hipStream_t>(stream);
+  const bool two = a.M > 16;
+  switch (groupsize) {
+    case 32: return two ? launch<32, 8, 2, 1, 4, 2, kPartial>(a) : launch<32, 8, 1, 1, 4, 2, kPartial>(a);
+    case 64: return two ? launch<64, 8, 2, 1, 4, 2, kPartial>(a) : launch<64, 8, 1, 1, 4, 2, kPartial>(a);
+    default: return two ? launch<128, 8, 2, 1, 4, 2, kPartial>(a) : launch<128, 8, 1, 1, 4, 2, kPartial>(a);
   }
 }

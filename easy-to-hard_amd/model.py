@@ -24,6 +24,7 @@ FUSED_DECODE = True
 # finer switches under FUSED_DECODE (both on by default; tests and measurements turn them off to compare)
 FUSE_GATE = True            # silu(w1 x) * w3 x as one int4 launch
 FUSE_ROPE_PROJECTION = True  # q|k|v projection + RoPE + cache write as one int4 launch
+DEFER_SPLIT_K = True         # wo / w2 hand float32 K-slice sums to the residual add + RMSNorm instead of combining them
 
 
 def _fusable(t: Tensor) -> bool:
@@ -130,6 +131,18 @@ def apply_rotary_emb(x: Tensor, freqs_cis: Tensor) -> Tensor:
     return torch.stack([re, im], dim=-1).flatten(3).type_as(x)
 
 
+def _project_deferred(lin, y2d: Tensor, lead_shape) -> Tensor:
+    """`lin(y)` for the fused path, y2d [rows, K] bfloat16.  Where the library would split K over several workgroups the
+    result comes back as float32 partial sums [slices, rows, N] for ops.add_rmsnorm to add, which spares the launch the
+    meeting of its slices; otherwise the projection itself, shaped [*lead_shape, N]."""
+    rows = y2d.shape[0]
+    if isinstance(lin, WeightOnlyInt4Linear) and y2d.dtype == torch.bfloat16:
+        slices = ops.int4_partial_slices(rows, lin)
+        if slices > 1:
+            return ops.int4_mm_partials(y2d, lin.weight, lin.groupsize, lin.scales_and_zeros, slices)
+    return lin(y2d.view(*lead_shape, -1))
+
+
 class Attention(nn.Module):
     def __init__(self, config: ModelArgs):
         super().__init__()
@@ -168,7 +181,9 @@ class Attention(nn.Module):
         return self.kv_cache is not None and self.freqs_table.shape[0] >= self.kv_cache.k_cache.shape[2]
 
     def forward(self, x: Tensor, freqs_cis: Optional[Tensor], mask: Optional[Tensor], input_pos: Optional[Tensor] = None,
-                fully_causal: bool = False) -> Tensor:
+                fully_causal: bool = False, defer_output: bool = False) -> Tensor:
+        """defer_output (fused decode step only): the output projection may come back as float32 partial sums over K
+        slices, to be added by the residual add + RMSNorm that follows (ops.add_rmsnorm takes either form)."""
         bsz, seqlen, _ = x.shape
         kv_size = self.n_local_heads * self.head_dim
         if self.can_fuse_decode(x, fully_causal):
@@ -187,6 +202,8 @@ class Attention(nn.Module):
                 q = ops.rope_kv_write(qkv, self.freqs_table, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos,
                                       self.n_head, self.n_local_heads, self.head_dim)
             y = ops.decode_attention(q, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, self.left_pad_mask_pos)
+            if defer_output:
+                return _project_deferred(self.wo, y.view(bsz, self.dim), (bsz, 1))
             return self.wo(y.view(bsz, 1, self.dim))
         if self._can_fuse_prefill_rope(x, input_pos, fully_causal):
             # many new tokens per sequence: rotation, head-major layout and cache write in one pass over qkv
@@ -240,7 +257,11 @@ class FeedForward(nn.Module):
             return False
         return not torch.compiler.is_compiling() and ops.int8_gate_supported(x, w1, w3)
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, defer_output: bool = False) -> Tensor:
+        if defer_output and self._gate_fusable(x):
+            y = ops.int4_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales_and_zeros,
+                                      self.w3.weight, self.w3.scales_and_zeros, self.w1.groupsize)
+            return _project_deferred(self.w2, y, x.shape[:-1])
         if self._gate_fusable_int8(x):
             y = ops.int8_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales, self.w3.weight, self.w3.scales)
             return self.w2(y.reshape(*x.shape[:-1], y.shape[-1]))
@@ -281,9 +302,9 @@ class TransformerBlock(nn.Module):
             normed = ops.rmsnorm(x, self.attention_norm.weight, self.attention_norm.eps)
         else:
             x, normed = ops.add_rmsnorm(x, delta, self.attention_norm.weight, self.attention_norm.eps)
-        attn = self.attention(normed, freqs_cis, mask, input_pos, fully_causal)
+        attn = self.attention(normed, freqs_cis, mask, input_pos, fully_causal, defer_output=DEFER_SPLIT_K)
         h, normed2 = ops.add_rmsnorm(x, attn, self.ffn_norm.weight, self.ffn_norm.eps)
-        return h, self.feed_forward(normed2)
+        return h, self.feed_forward(normed2, defer_output=DEFER_SPLIT_K)
 
 
 class Transformer(nn.Module):

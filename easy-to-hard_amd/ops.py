@@ -396,8 +396,49 @@ def rmsnorm(x, weight, eps):
     return y
 
 
+def int4_partial_slices(rows: int, lin) -> int:
+    """Number of K slices the library splits `lin` (a WeightOnlyInt4Linear) into for `rows` rows of x when its result is
+    handed on as partial sums; 0 where that form does not apply (more than 64 rows, padded K, other geometries)."""
+    if getattr(lin, "padding", False) and getattr(lin, "origin_in_features", lin.in_features) != lin.in_features:
+        return 0
+    if lin.inner_k_tiles != 8 or rows < 1 or rows > 64:
+        return 0
+    s = _lib.load().e2h_int4_mm_partial_slices(rows, lin.out_features, lin.in_features, lin.groupsize, lin.inner_k_tiles)
+    return s if s > 0 else 0
+
+
+def int4_mm_partials(x, weight_int4pack, groupsize, scales_and_zeros, slices):
+    """x [M, K] bf16 -> float32 [slices, M, N]: the sums over `slices` contiguous parts of K, left for add_rmsnorm to add
+    (in slice order) instead of meeting inside the matmul launch."""
+    _need_gpu(x, weight_int4pack, scales_and_zeros)
+    assert x.dtype == torch.bfloat16 and x.dim() == 2
+    x = x.contiguous()
+    n = weight_int4pack.shape[0] * 8
+    m, k = x.shape
+    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    rc = _lib_for(x).e2h_int4_mm_partials(_ptr(x), _ptr(weight_int4pack), _ptr(scales_and_zeros), _ptr(out), m, n, k, groupsize,
+                                          weight_int4pack.shape[3] * 2, slices, _stream(x))
+    _lib.check(rc, "e2h_int4_mm_partials")
+    return out
+
+
 def add_rmsnorm(x, delta, weight, eps):
-    """h = bf16(x + delta); returns (h, RMSNorm(h)) -- the residual add and the following norm in one kernel."""
+    """h = bf16(x + delta); returns (h, RMSNorm(h)) -- the residual add and the following norm in one kernel.  `delta` is
+    either a bfloat16 tensor of x's shape or float32 partial sums [slices, rows, dim] from int4_mm_partials, in which case
+    the term added is bf16(sum over slices, in order)."""
+    if delta.dtype == torch.float32:
+        _need_gpu(x, delta, weight)
+        assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and delta.dim() == 3 and delta.is_contiguous()
+        x = x.contiguous()
+        dim = x.shape[-1]
+        rows = x.numel() // dim
+        assert delta.shape[1] == rows and delta.shape[2] == dim
+        h = torch.empty_like(x)
+        y = torch.empty_like(x)
+        rc = _lib_for(x).e2h_add_rmsnorm_partials(_ptr(x), _ptr(delta), delta.shape[0], _ptr(weight), _ptr(h), _ptr(y), rows, dim,
+                                                  float(eps), _stream(x))
+        _lib.check(rc, "e2h_add_rmsnorm_partials")
+        return h, y
     _need_gpu(x, delta, weight)
     assert x.dtype == torch.bfloat16 and delta.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape == delta.shape
     x, delta = x.contiguous(), delta.contiguous()

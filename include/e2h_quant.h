@@ -211,6 +211,21 @@ int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *y, int64_t 
 int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *weight, uint16_t *h_out,
                     uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream);
 
+/* The wo / w2 projection of a decoder block and the residual add + RMSNorm that consumes it (TransformerBlock.forward,
+ * reference models/model.py:279-283; the projections are WeightOnlyInt4Linear.forward, models/quantize.py:445-453), as a
+ * pair of launches that never meet inside the matmul: for up to 64 rows of x, inner_k_tiles 8 and group size <= 128,
+ * e2h_int4_mm_partials writes the float32 sums of `slices` contiguous parts of K to partials [slices, m, n] (row-major),
+ * and e2h_add_rmsnorm_partials forms delta = bf16(partials[0] + partials[1] + ... in that order) -- bit for bit the
+ * value e2h_int4_mm stores for the same operands -- before h_out = bf16(x + delta), y = RMSNorm(h_out).
+ * e2h_int4_mm_partial_slices returns the number of slices the library uses for a shape (>= 1; it depends on the shape
+ * and on e2h_set_option only), or a negative status for shapes this form does not take; e2h_int4_mm_partials rejects
+ * any other `slices`.  No workspace is involved. */
+int e2h_int4_mm_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles);
+int e2h_int4_mm_partials(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, float *partials,
+                         int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, int slices, void *stream);
+int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *weight,
+                             uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream);
+
 /* apply_rotary_emb (reference :400-412) on the q and k parts of a fused qkv row + KVCache.update (:121-129) for
  * one new token per sequence.  qkv [batch, (n_head + 2 n_kv_head) * head_dim]; freqs_cis [positions, head_dim/2, 2]
  * bf16 (cos, sin); q_out [batch, n_head, head_dim]; caches as above, written at *input_pos. */

@@ -185,3 +185,92 @@ def test_reward_model_loader_with_on_the_fly_int8(tmp_path):
     assert got.shape == (3, 24)
     assert float((got - want).abs().max()) <= 1e-1 * float(want.abs().max())
     assert torch.equal(model_score(direct, ids), torch.zeros_like(got, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("m,n,k,g", [(32, 4096, 4096, 128), (1, 4096, 4096, 128), (5, 4096, 11008, 128), (33, 1024, 2048, 64), (64, 8192, 8192, 64),
+                                      (17, 264, 1024, 32), (32, 12288, 4096, 128)])
+def test_partial_sums_handed_to_the_norm_equal_the_combined_matmul(m, n, k, g):
+    """e2h_int4_mm_partials + e2h_add_rmsnorm_partials against e2h_int4_mm + e2h_add_rmsnorm on the same operands: the
+    slices are added in slice order in both forms, so the residual stream and the normed output are equal bit for bit;
+    the partial sums themselves add up (in float32, in order) to a value that rounds to the matmul's output."""
+    w = randn_bf16((n, k), std=0.02, seed=n + k).to(DEV)
+    packed, sz = e2h.prepare_int4_weight_and_scales_and_zeros(w, g, 8)
+    lin = e2h.WeightOnlyInt4Linear(k, n, bias=False, groupsize=g, inner_k_tiles=8, padding=False).to(DEV)
+    lin.weight, lin.scales_and_zeros = packed, sz
+    x = randn_bf16((m, k), seed=m).to(DEV)
+    resid = randn_bf16((m, n), seed=m + 1).to(DEV)
+    gamma = (1 + 0.1 * torch.randn(n, generator=torch.Generator().manual_seed(3))).to(torch.bfloat16).to(DEV)
+    slices = ops.int4_partial_slices(m, lin)
+    assert slices >= 1
+    parts = ops.int4_mm_partials(x, packed, g, sz, slices)
+    assert parts.shape == (slices, m, n) and parts.dtype == torch.float32
+    y = ops.int4_mm_direct(x, packed, g, sz)
+    total = parts[0].clone()
+    for s in range(1, slices):
+        total += parts[s]
+    assert torch.equal(total.to(torch.bfloat16), y)
+    h1, n1 = ops.add_rmsnorm(resid, y, gamma, 1e-5)
+    h2, n2 = ops.add_rmsnorm(resid, parts, gamma, 1e-5)
+    assert torch.equal(h1, h2) and torch.equal(n1, n2)
+
+
+def test_partial_sum_form_is_refused_where_it_does_not_apply():
+    lin = e2h.WeightOnlyInt4Linear(1024, 64, bias=False, groupsize=128, inner_k_tiles=4, padding=False)
+    assert ops.int4_partial_slices(8, lin) == 0                     # inner_k_tiles 4
+    lin8 = e2h.WeightOnlyInt4Linear(1024, 64, bias=False, groupsize=128, inner_k_tiles=8, padding=False)
+    assert ops.int4_partial_slices(65, lin8) == 0 and ops.int4_partial_slices(0, lin8) == 0
+    assert ops.int4_partial_slices(8, lin8) >= 1
+    from easy_to_hard_amd import _lib
+    lib = _lib.load()
+    assert lib.e2h_int4_mm_partial_slices(8, 64, 1024, 256, 8) < 0    # group size 256
+    assert lib.e2h_int4_mm_partial_slices(8, 60, 1024, 128, 8) < 0    # N % 8
+    x = randn_bf16((8, 1024), seed=1).to(DEV)
+    w = randn_bf16((64, 1024), std=0.02, seed=2).to(DEV)
+    packed, sz = e2h.prepare_int4_weight_and_scales_and_zeros(w, 128, 8)
+    want = ops.int4_partial_slices(8, lin8)
+    out = torch.empty((want + 1, 8, 64), dtype=torch.float32, device=DEV)
+    rc = lib.e2h_int4_mm_partials(ops._ptr(x), ops._ptr(packed), ops._ptr(sz), ops._ptr(out), 8, 64, 1024, 128, 8, want + 1, ops._stream(x))
+    assert rc < 0                                                   # a slice count other than the library's own
+
+
+@pytest.mark.parametrize("bsz", [32, 5])
+def test_decode_step_with_deferred_slices_equals_the_step_without(bsz, monkeypatch):
+    """The fused decode step with wo / w2 handing partial sums to the norms (model.DEFER_SPLIT_K) against the same step with
+    the matmuls combining their slices themselves, on two layers of the 7B shape (K = 4096 and 11008 are long enough for
+    the library to split): identical logits, eagerly and from a HIP graph."""
+    import easy_to_hard_amd.model as model_mod
+    from easy_to_hard_amd.model import ModelArgs, random_quantized_transformer
+
+    cfg = ModelArgs.from_name("7B")
+    cfg.n_layer = 2
+    model = random_quantized_transformer(cfg, "int4", 128, device=DEV, seed=7)
+    t = 7
+    prompt = torch.randint(0, cfg.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(4)).to(DEV)
+    calls = []
+    real = ops.int4_mm_partials
+    monkeypatch.setattr(ops, "int4_mm_partials", lambda *a, **k: (calls.append(a[-1]), real(*a, **k))[1])
+    logits = {}
+    for defer in (False, True):
+        model_mod.DEFER_SPLIT_K = defer
+        try:
+            model.max_seq_length = -1
+            model.setup_caches(bsz, 32)
+            cur = prefill(model, prompt, torch.arange(0, t, device=DEV))
+            out = []
+            for i in range(3):
+                lg = model(cur, torch.tensor([t + i], device=DEV))
+                out.append(lg[:, -1].clone())
+                cur = torch.argmax(lg[:, -1].float(), dim=-1, keepdim=True)
+            logits[defer] = torch.stack(out)
+            if defer:
+                assert calls and min(calls) > 1          # both projections of both layers took the partial-sum form
+                stepper = GraphedDecodeStep(model, bsz, DEV)
+                prefill(model, prompt, torch.arange(0, t, device=DEV))
+                first = torch.argmax(logits[False][0].float(), dim=-1, keepdim=True)
+                tok = stepper.step(first, torch.tensor([t + 1], device=DEV)).clone()
+                assert torch.equal(tok, torch.argmax(logits[False][1].float(), dim=-1, keepdim=True))
+            else:
+                assert not calls
+        finally:
+            model_mod.DEFER_SPLIT_K = True
+    assert torch.equal(logits[True], logits[False])
