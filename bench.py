@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-Workload (default): BASELINE config "random-init Llama-2-7B-architecture model with int4 g128 weight-only
+Workload (default): the headline configuration, "random-init Llama-2-7B-architecture model with int4 g128 weight-only
 linears, batch 32, prompt 256, 512 greedy-decoded tokens, bf16 KV cache".  One step = one decode step of the whole
 batch (129 dequant-GEMV launches -- w1 and w3 of a block share one gated launch -- plus decode attention, norms,
 RoPE), replayed from a HIP graph.  The timed steps sit at cache positions spread evenly over the whole decode, so

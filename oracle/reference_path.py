@@ -1,6 +1,6 @@
 """The reference's CPU execution path for a weight-only quantized linear, restated with torch CPU ops.
 
-TEST / BASELINE INFRASTRUCTURE ONLY (same rule as quant_oracle.py): used as the timed CPU baseline of the
+TEST AND CPU-BASELINE INFRASTRUCTURE ONLY (same rule as quant_oracle.py): used as the timed CPU baseline of the
 benchmark and as a cross-check in tests, never by the shipped package.
 
   int8:  F.linear(x, weight.to(x.dtype)) * scales                       reference models/quantize.py:428-429

@@ -175,7 +175,7 @@ def _check_int8(x, q, s, q_d, s_d):
 
 
 def test_int8_mm_config1():
-    # BASELINE config 1: 4096x4096 weight ~N(0, 0.02), x [8, 4096] ~N(0, 1), seed 1234
+    # benchmark configuration 1: 4096x4096 weight ~N(0, 0.02), x [8, 4096] ~N(0, 1), seed 1234
     q, s, q_d, s_d = _int8_case(4096, 4096)
     x = randn_bf16((8, 4096), seed=1235)
     y, err = _check_int8(x, q, s, q_d, s_d)
