@@ -34,7 +34,9 @@ _SIGNATURES = {
     "e2h_add_rmsnorm": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "e2h_int4_mm_partial_slices": (c_int, [c_int64, c_int64, c_int64, c_int, c_int]),
     "e2h_int4_mm_partials": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, c_int, _P]),
-    "e2h_add_rmsnorm_partials": (c_int, [_P, _P, c_int, _P, _P, _P, c_int64, c_int64, c_float, _P]),
+    "e2h_int8_mm_partial_slices": (c_int, [c_int64, c_int64, c_int64]),
+    "e2h_int8_mm_partials": (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),
+    "e2h_add_rmsnorm_partials": (c_int, [_P, _P, c_int, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
     "e2h_rope_kv_write": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
     "e2h_rope_kv_write_seq": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, _P]),
     "e2h_silu_mul": (c_int, [_P, _P, _P, c_int64, _P]),

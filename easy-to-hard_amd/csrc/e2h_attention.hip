@@ -361,6 +361,7 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ delta,
                                                         const float *__restrict__ psum, int slices,
+                                                        const uint16_t *__restrict__ col_scales,
                                                         const uint16_t *__restrict__ w, uint16_t *__restrict__ h_out,
                                                         uint16_t *__restrict__ y, int dim, float eps) {
   constexpr int kPieces = 2, kStride = BLOCK * 8, kWaves = BLOCK / 64;
@@ -369,7 +370,8 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
   const uint16_t *xr = x + row * dim;
   const uint16_t *dr_row = delta ? delta + row * dim : nullptr;
   // psum: the term to add arrives as float32 partial sums [slices][rows][dim] of a matmul split along K; the term is
-  // bf16(p[0] + p[1] + .. in slice order), the value the matmul's own combine step would have stored
+  // bf16(p[0] + p[1] + .. in slice order), the value the matmul's own combine step would have stored -- with
+  // col_scales (int8 weights) bf16(that * scale[column]), the two roundings of the int8 linear
   const size_t slice_floats = static_cast<size_t>(gridDim.x) * dim;
   const float *pr = psum ? psum + row * dim : nullptr;
   auto sum_slices = [&](int i) {
@@ -390,6 +392,16 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
     for (int s2 = kMaxSlices; s2 < slices; ++s2) {
       a += *reinterpret_cast<const f32x4_t *>(pr + s2 * slice_floats + i);
       b += *reinterpret_cast<const f32x4_t *>(pr + s2 * slice_floats + i + 4);
+    }
+    if (col_scales) {
+      const u32x4_t cs = *reinterpret_cast<const u32x4_t *>(col_scales + i);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        a[2 * j] = bf16_round(a[2 * j]) * __builtin_bit_cast(float, cs[j] << 16);
+        a[2 * j + 1] = bf16_round(a[2 * j + 1]) * __builtin_bit_cast(float, cs[j] & 0xFFFF0000u);
+        b[2 * j] = bf16_round(b[2 * j]) * __builtin_bit_cast(float, cs[2 + j] << 16);
+        b[2 * j + 1] = bf16_round(b[2 * j + 1]) * __builtin_bit_cast(float, cs[2 + j] & 0xFFFF0000u);
+      }
     }
     u32x4_t d;
     d[0] = static_cast<uint32_t>(f32_to_bf16_rne(a[0])) | (static_cast<uint32_t>(f32_to_bf16_rne(a[1])) << 16);
@@ -549,14 +561,14 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
 }
 
 // few rows (decode): 512 threads so that a 4096-wide row is one piece per thread; many rows: 256-thread workgroups
-void launch_rmsnorm(const uint16_t *x, const uint16_t *delta, const float *psum, int slices, const uint16_t *w, uint16_t *h_out, uint16_t *y,
-                    int64_t rows, int64_t dim, float eps, hipStream_t stream) {
+void launch_rmsnorm(const uint16_t *x, const uint16_t *delta, const float *psum, int slices, const uint16_t *col_scales, const uint16_t *w,
+                    uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps, hipStream_t stream) {
   if (rows <= 512 && dim >= 4096)
-    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(static_cast<unsigned>(rows)), dim3(512), 0, stream, x, delta, psum, slices, w, h_out, y,
-                       static_cast<int>(dim), eps);
+    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(static_cast<unsigned>(rows)), dim3(512), 0, stream, x, delta, psum, slices, col_scales, w, h_out,
+                       y, static_cast<int>(dim), eps);
   else
-    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, x, delta, psum, slices, w, h_out, y,
-                       static_cast<int>(dim), eps);
+    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, x, delta, psum, slices, col_scales, w, h_out,
+                       y, static_cast<int>(dim), eps);
 }
 
 template <int D, int NW>
@@ -617,7 +629,7 @@ extern "C" int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *
   if (!x || !weight || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, nullptr, nullptr, 0, weight, nullptr, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, nullptr, nullptr, 0, nullptr, weight, nullptr, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 
@@ -626,16 +638,18 @@ extern "C" int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const u
   if (!x || !delta || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(delta) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, delta, nullptr, 0, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, delta, nullptr, 0, nullptr, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 
-extern "C" int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *weight, uint16_t *h_out,
-                                        uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream) {
+extern "C" int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *col_scales,
+                                        const uint16_t *weight, uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps,
+                                        void *stream) {
   if (!x || !partials || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX || slices < 1 || slices > 64) return E2H_ERR_BAD_SHAPE;
-  if (!aligned16(x) || !aligned16(partials) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, nullptr, partials, slices, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  if (!aligned16(x) || !aligned16(partials) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y) || (col_scales && !aligned16(col_scales)))
+    return E2H_ERR_MISALIGNED;
+  launch_rmsnorm(x, nullptr, partials, slices, col_scales, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 

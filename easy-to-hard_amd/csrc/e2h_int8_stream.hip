@@ -56,7 +56,10 @@ struct WeightRegs8 {
 //   bfloat16 output is rotated in float32 by the angle of position input_pos[0] (interleaved pairs, reference
 //   models/model.py:400-412); q goes to q_out [B, H, D], k and v into the caches [B, Hkv, S, D] at that position
 //   (KVCache.update, reference models/model.py:94-104).
-enum Epilogue8 { kPlain8 = 0, kGate8 = 1, kRope8 = 2 };
+// kPartial8: the workgroup's float32 sums over its K slice (unscaled) go to slice blockIdx.y of a row-major [S][M][N]
+// array and the launch ends there; the residual add + RMSNorm that follows adds the slices in order and applies the
+// column scales with the reference's two roundings.
+enum Epilogue8 { kPlain8 = 0, kGate8 = 1, kRope8 = 2, kPartial8 = 3 };
 
 struct Rope8Args {
   const uint16_t *freqs;     // [>= S, D/2, 2] bf16 (cos, sin)
@@ -265,6 +268,23 @@ __global__ __launch_bounds__(64 * WN * WK) void int8_stream_mm_kernel(const uint
     }
   }
 
+  if constexpr (EPI == kPartial8) {
+    if (kg != 0) return;
+    float *out = ws_partial + static_cast<size_t>(ks) * M * N;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const int n = 16 * (tile16_0 + t) + c;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = m_base + 16 * mt + 4 * b + r;
+          if (n < N && m < M) out[static_cast<size_t>(m) * N + n] = acc[t][mt][r];
+        }
+    }
+    return;
+  }
+
   if (S > 1) {
     const size_t tile_floats = static_cast<size_t>(WN) * kSlots * 64;
     const size_t wg_tile = static_cast<size_t>(blockIdx.z) * gridDim.x + blockIdx.x;
@@ -403,6 +423,36 @@ int launch8(const Args8 &a) {
 constexpr size_t kTicketBytes8 = 64 * 1024;
 constexpr int kCUs8 = 256;
 
+// K slices for the 16- and 32-row decode shapes (4 column waves x 2 k-groups), as in the int4 kernel
+inline int decode_k_slices8(int blocks, int nchunks) {
+  int s = 1;
+  while (s < 4 && blocks * s * 2 <= kCUs8 && nchunks / (2 * s * 2) >= 4) s *= 2;
+  return s;
+}
+
+// rows per workgroup (in 16-row tiles) of the decode shapes, 0 where a call takes another kernel
+inline int decode_row_tiles8(int M, int N) {
+  const int tiles16 = (N + 15) / 16;
+  if (M <= 16) return 1;
+  if (M <= 32) return 2;
+  if (M <= 64 && (tiles16 + 3) / 4 < kCUs8) return 2;
+  return 0;
+}
+
+int partial_slices8_for(int64_t m, int64_t n, int64_t k) {
+  if (m < 1 || m > 64 || n < 8 || (n % 8) != 0 || k < 128 || (k % 128) != 0 || n > INT32_MAX || k > INT32_MAX || n * k >= (int64_t{1} << 32))
+    return E2H_ERR_BAD_SHAPE;
+  const int mt = decode_row_tiles8(static_cast<int>(m), static_cast<int>(n));
+  if (mt == 0) return E2H_ERR_BAD_SHAPE;
+  const int m_chunks = static_cast<int>((m + 16 * mt - 1) / (16 * mt));
+  const int tiles16 = static_cast<int>((n + 15) / 16);
+  const int nchunks = static_cast<int>(k / kChunk);
+  int s = decode_k_slices8(((tiles16 + 3) / 4) * m_chunks, nchunks);
+  if (options().int8_k_slices > 0) s = options().int8_k_slices;
+  if (s > nchunks) s = nchunks;
+  return s;
+}
+
 }  // namespace
 
 // Streaming int8 matmul; the caller has checked pointers and that K % 128 == 0 with 16-byte aligned x and q.
@@ -425,8 +475,7 @@ int int8_stream_mm(const uint16_t *x, const int8_t *q, const uint16_t *scales, u
     t = (static_cast<long long>((tiles16 + 7) / 8) * m_chunks >= kCUs8) ? 2 : 1;
   } else {
     const int blocks = ((tiles16 + 3) / 4) * m_chunks;
-    if (have_ws)
-      while (s < 4 && blocks * s * 2 <= kCUs8 && nchunks / (2 * s * wk) >= 4) s *= 2;
+    if (have_ws) s = decode_k_slices8(blocks, nchunks);
     // more column blocks than CUs: two column tiles per wave halve the number of workgroups and cost less than a
     // second round of them (measured: 32000 x 4096 at 32 rows 42.4 instead of 46.6 us, at 16 rows 34.6 instead of
     // 38.2; 12288 x 4096 at 64 rows, two slabs, 30.1 instead of 37.3)
@@ -510,4 +559,23 @@ extern "C" int e2h_int8_mm_rope_kv(const uint16_t *x, const int8_t *q, const uin
   a.M = static_cast<int>(batch); a.N = static_cast<int>(n); a.K = static_cast<int>(k); a.S = 1;
   a.stream = static_cast<hipStream_t>(stream);
   return a.M <= 16 ? launch8<1, 1, 4, 2, kRope8>(a) : launch8<2, 1, 4, 2, kRope8>(a);
+}
+
+extern "C" int e2h_int8_mm_partial_slices(int64_t m, int64_t n, int64_t k) { return e2h::partial_slices8_for(m, n, k); }
+
+extern "C" int e2h_int8_mm_partials(const uint16_t *x, const int8_t *q, float *partials, int64_t m, int64_t n, int64_t k, int slices,
+                                    void *stream) {
+  using namespace e2h;
+  if (!x || !q || !partials) return E2H_ERR_NULL_POINTER;
+  const int want = partial_slices8_for(m, n, k);
+  if (want < 0) return want;
+  if (slices != want) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(q) || (reinterpret_cast<uintptr_t>(partials) & 3u)) return E2H_ERR_MISALIGNED;
+  Args8 a;
+  a.x = x; a.q = q; a.scales = nullptr; a.q2 = nullptr; a.scales2 = nullptr; a.y = nullptr;
+  a.rope = Rope8Args{};
+  a.ws_partial = partials; a.ws_ticket = nullptr;
+  a.M = static_cast<int>(m); a.N = static_cast<int>(n); a.K = static_cast<int>(k); a.S = slices;
+  a.stream = static_cast<hipStream_t>(stream);
+  return decode_row_tiles8(a.M, a.N) == 1 ? launch8<1, 1, 4, 2, kPartial8>(a) : launch8<2, 1, 4, 2, kPartial8>(a);
 }

@@ -140,6 +140,10 @@ def _project_deferred(lin, y2d: Tensor, lead_shape) -> Tensor:
         slices = ops.int4_partial_slices(rows, lin)
         if slices > 1:
             return ops.int4_mm_partials(y2d, lin.weight, lin.groupsize, lin.scales_and_zeros, slices)
+    if isinstance(lin, WeightOnlyInt8Linear) and y2d.dtype == torch.bfloat16 and lin.scales.dtype == torch.bfloat16:
+        slices = ops.int8_partial_slices(rows, lin)
+        if slices > 1:
+            return ops.int8_mm_partials(y2d, lin.weight, lin.scales, slices)
     return lin(y2d.view(*lead_shape, -1))
 
 
@@ -258,6 +262,9 @@ class FeedForward(nn.Module):
         return not torch.compiler.is_compiling() and ops.int8_gate_supported(x, w1, w3)
 
     def forward(self, x: Tensor, defer_output: bool = False) -> Tensor:
+        if defer_output and self._gate_fusable_int8(x):
+            y = ops.int8_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales, self.w3.weight, self.w3.scales)
+            return _project_deferred(self.w2, y, x.shape[:-1])
         if defer_output and self._gate_fusable(x):
             y = ops.int4_mm_silu_gate(x.reshape(-1, x.shape[-1]), self.w1.weight, self.w1.scales_and_zeros,
                                       self.w3.weight, self.w3.scales_and_zeros, self.w1.groupsize)

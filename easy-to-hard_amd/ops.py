@@ -422,10 +422,42 @@ def int4_mm_partials(x, weight_int4pack, groupsize, scales_and_zeros, slices):
     return out
 
 
+def int8_partial_slices(rows: int, lin) -> int:
+    """As int4_partial_slices, for a WeightOnlyInt8Linear."""
+    if rows < 1 or rows > 64 or lin.in_features % 128 != 0 or lin.out_features % 8 != 0:
+        return 0
+    s = _lib.load().e2h_int8_mm_partial_slices(rows, lin.out_features, lin.in_features)
+    return s if s > 0 else 0
+
+
+class ScaledPartials:
+    """float32 K-slice sums [slices, rows, N] of an int8 matmul together with the column scales that turn them into the
+    linear's output; add_rmsnorm takes it in place of `delta`."""
+
+    def __init__(self, partials, scales):
+        self.partials, self.scales = partials, scales
+
+
+def int8_mm_partials(x, q, scales, slices):
+    """x [M, K] bf16, q int8 [N, K] -> ScaledPartials (unscaled float32 sums over `slices` parts of K + the bf16 scales)."""
+    _need_gpu(x, q, scales)
+    assert x.dtype == torch.bfloat16 and x.dim() == 2 and q.dtype == torch.int8 and scales.dtype == torch.bfloat16
+    x = x.contiguous()
+    m, k = x.shape
+    n = q.shape[0]
+    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    rc = _lib_for(x).e2h_int8_mm_partials(_ptr(x), _ptr(q), _ptr(out), m, n, k, slices, _stream(x))
+    _lib.check(rc, "e2h_int8_mm_partials")
+    return ScaledPartials(out, scales)
+
+
 def add_rmsnorm(x, delta, weight, eps):
     """h = bf16(x + delta); returns (h, RMSNorm(h)) -- the residual add and the following norm in one kernel.  `delta` is
-    either a bfloat16 tensor of x's shape or float32 partial sums [slices, rows, dim] from int4_mm_partials, in which case
-    the term added is bf16(sum over slices, in order)."""
+    either a bfloat16 tensor of x's shape, or float32 partial sums [slices, rows, dim] from int4_mm_partials, in which case
+    the term added is bf16(sum over slices, in order), or the ScaledPartials of int8_mm_partials."""
+    col_scales = None
+    if isinstance(delta, ScaledPartials):
+        delta, col_scales = delta.partials, delta.scales
     if delta.dtype == torch.float32:
         _need_gpu(x, delta, weight)
         assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and delta.dim() == 3 and delta.is_contiguous()
@@ -435,8 +467,8 @@ def add_rmsnorm(x, delta, weight, eps):
         assert delta.shape[1] == rows and delta.shape[2] == dim
         h = torch.empty_like(x)
         y = torch.empty_like(x)
-        rc = _lib_for(x).e2h_add_rmsnorm_partials(_ptr(x), _ptr(delta), delta.shape[0], _ptr(weight), _ptr(h), _ptr(y), rows, dim,
-                                                  float(eps), _stream(x))
+        rc = _lib_for(x).e2h_add_rmsnorm_partials(_ptr(x), _ptr(delta), delta.shape[0], _ptr(col_scales) if col_scales is not None else None,
+                                                  _ptr(weight), _ptr(h), _ptr(y), rows, dim, float(eps), _stream(x))
         _lib.check(rc, "e2h_add_rmsnorm_partials")
         return h, y
     _need_gpu(x, delta, weight)

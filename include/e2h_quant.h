@@ -219,12 +219,19 @@ int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *we
  * value e2h_int4_mm stores for the same operands -- before h_out = bf16(x + delta), y = RMSNorm(h_out).
  * e2h_int4_mm_partial_slices returns the number of slices the library uses for a shape (>= 1; it depends on the shape
  * and on e2h_set_option only), or a negative status for shapes this form does not take; e2h_int4_mm_partials rejects
- * any other `slices`.  No workspace is involved. */
+ * any other `slices`.  No workspace is involved.
+ * The int8 pair (WeightOnlyInt8Linear.forward, models/quantize.py:428-429; K % 128 == 0, 16-byte aligned rows) hands on the
+ * unscaled sums; col_scales [n] bf16 (NULL for int4) makes the consumer form delta = bf16(bf16(sum) * scale[column]), the
+ * linear's two roundings. */
 int e2h_int4_mm_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles);
 int e2h_int4_mm_partials(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, float *partials,
                          int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, int slices, void *stream);
-int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *weight,
-                             uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream);
+int e2h_int8_mm_partial_slices(int64_t m, int64_t n, int64_t k);
+int e2h_int8_mm_partials(const uint16_t *x, const int8_t *q, float *partials, int64_t m, int64_t n, int64_t k, int slices,
+                         void *stream);
+int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *col_scales,
+                             const uint16_t *weight, uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps,
+                             void *stream);
 
 /* apply_rotary_emb (reference :400-412) on the q and k parts of a fused qkv row + KVCache.update (:121-129) for
  * one new token per sequence.  qkv [batch, (n_head + 2 n_kv_head) * head_dim]; freqs_cis [positions, head_dim/2, 2]

@@ -214,6 +214,26 @@ def test_partial_sums_handed_to_the_norm_equal_the_combined_matmul(m, n, k, g):
     assert torch.equal(h1, h2) and torch.equal(n1, n2)
 
 
+@pytest.mark.parametrize("m,n,k", [(32, 4096, 4096), (1, 4096, 4096), (5, 4096, 11008), (64, 1024, 2048), (17, 264, 1024)])
+def test_int8_partial_sums_handed_to_the_norm_equal_the_combined_matmul(m, n, k):
+    """The int8 pair: unscaled K-slice sums + column scales into the norm against e2h_int8_mm + e2h_add_rmsnorm."""
+    w = randn_bf16((n, k), std=0.02, seed=n + k + 1).to(DEV)
+    q, scales, _ = e2h.dynamically_quantize_per_channel(w.float(), -128, 127, torch.int8)
+    lin = e2h.WeightOnlyInt8Linear(k, n).to(DEV)
+    lin.load_state_dict({"weight": q, "scales": scales})
+    x = randn_bf16((m, k), seed=m + 7).to(DEV)
+    resid = randn_bf16((m, n), seed=m + 8).to(DEV)
+    gamma = (1 + 0.1 * torch.randn(n, generator=torch.Generator().manual_seed(5))).to(torch.bfloat16).to(DEV)
+    slices = ops.int8_partial_slices(m, lin)
+    assert slices >= 1
+    parts = ops.int8_mm_partials(x, lin.weight, lin.scales, slices)
+    assert parts.partials.shape == (slices, m, n)
+    y = ops.int8_mm_direct(x, lin.weight, lin.scales)
+    h1, n1 = ops.add_rmsnorm(resid, y, gamma, 1e-5)
+    h2, n2 = ops.add_rmsnorm(resid, parts, gamma, 1e-5)
+    assert torch.equal(h1, h2) and torch.equal(n1, n2)
+
+
 def test_partial_sum_form_is_refused_where_it_does_not_apply():
     lin = e2h.WeightOnlyInt4Linear(1024, 64, bias=False, groupsize=128, inner_k_tiles=4, padding=False)
     assert ops.int4_partial_slices(8, lin) == 0                     # inner_k_tiles 4
@@ -233,8 +253,9 @@ def test_partial_sum_form_is_refused_where_it_does_not_apply():
     assert rc < 0                                                   # a slice count other than the library's own
 
 
+@pytest.mark.parametrize("mode", ["int4", "int8"])
 @pytest.mark.parametrize("bsz", [32, 5])
-def test_decode_step_with_deferred_slices_equals_the_step_without(bsz, monkeypatch):
+def test_decode_step_with_deferred_slices_equals_the_step_without(bsz, mode, monkeypatch):
     """The fused decode step with wo / w2 handing partial sums to the norms (model.DEFER_SPLIT_K) against the same step with
     the matmuls combining their slices themselves, on two layers of the 7B shape (K = 4096 and 11008 are long enough for
     the library to split): identical logits, eagerly and from a HIP graph."""
@@ -243,12 +264,13 @@ def test_decode_step_with_deferred_slices_equals_the_step_without(bsz, monkeypat
 
     cfg = ModelArgs.from_name("7B")
     cfg.n_layer = 2
-    model = random_quantized_transformer(cfg, "int4", 128, device=DEV, seed=7)
+    model = random_quantized_transformer(cfg, mode, 128, device=DEV, seed=7)
     t = 7
     prompt = torch.randint(0, cfg.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(4)).to(DEV)
     calls = []
-    real = ops.int4_mm_partials
-    monkeypatch.setattr(ops, "int4_mm_partials", lambda *a, **k: (calls.append(a[-1]), real(*a, **k))[1])
+    name = mode + "_mm_partials"
+    real = getattr(ops, name)
+    monkeypatch.setattr(ops, name, lambda *a, **k: (calls.append(a[-1]), real(*a, **k))[1])
     logits = {}
     for defer in (False, True):
         model_mod.DEFER_SPLIT_K = defer
