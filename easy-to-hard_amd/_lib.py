@@ -46,6 +46,16 @@ _SIGNATURES = {
     "e2h_int8_mm_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, _P]),
     "e2h_int8_mm_rope_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
     "e2h_int4_mm_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P]),
+    "e2h_int4_staged_bytes": (c_int64, [c_int64, c_int64]),
+    "e2h_int4_stage_x": (c_int, [_P, _P, c_int64, c_int64, _P]),
+    "e2h_int4_mm_staged_supported": (c_int, [c_int64, c_int64, c_int64, c_int, c_int]),
+    "e2h_int4_mm_staged": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),
+    "e2h_int4_mm_staged_partial_slices": (c_int, [c_int64, c_int64, c_int64, c_int]),
+    "e2h_int4_mm_staged_partials": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P]),
+    "e2h_int4_mm_staged_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),
+    "e2h_int4_mm_staged_rope_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, _P]),
+    "e2h_add_rmsnorm_staged": (c_int, [_P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
+    "e2h_decode_attention_staged": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, _P]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

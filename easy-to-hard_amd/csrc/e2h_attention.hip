@@ -7,6 +7,7 @@
 // (models/model.py: KVCache.update :121-129, Attention.forward :310-349, RMSNorm :363-377, apply_rotary_emb
 // :400-412, FeedForward.forward :359-360; decode loop inference_generate.py:110-157).
 #include "e2h_common.h"
+#include "e2h_staged.h"
 
 namespace e2h {
 namespace {
@@ -29,7 +30,7 @@ template <int D, int REP, int NW>
 __global__ __launch_bounds__(64 * NW) void decode_attention_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
                                                                const uint16_t *__restrict__ vc, uint16_t *__restrict__ out,
                                                                const int64_t *__restrict__ input_pos, const int64_t *__restrict__ left_pad,
-                                                               int H, int Hkv, int S, float scale) {
+                                                               int H, int Hkv, int S, float scale, StagedOut staged) {
   constexpr int LPP = D / 8;        // lanes per position
   constexpr int PPL = 64 / LPP;     // positions per wave-wide load
   constexpr int UNR = 4;            // loads in flight per wave
@@ -173,7 +174,9 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_kernel(const uint16_
       l += sh_l[w][r] * c;
       a += sh_acc[w][r][d] * c;
     }
-    out[(static_cast<size_t>(b) * H + hk * REP + r) * D + d] = f32_to_bf16_rne(a / l);
+    const uint16_t o = f32_to_bf16_rne(a / l);
+    if (out) out[(static_cast<size_t>(b) * H + hk * REP + r) * D + d] = o;
+    if (staged.frag) staged_store_run16(staged, b, (hk * REP + r) * D + d, o);  // whole aligned 16-lane groups get here together
   }
 }
 
@@ -197,7 +200,7 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
                                                                        const uint16_t *__restrict__ vc, uint16_t *__restrict__ out,
                                                                        const int64_t *__restrict__ input_pos,
                                                                        const int64_t *__restrict__ left_pad, int H, int Hkv, int S, int rep,
-                                                                       float scale) {
+                                                                       float scale, StagedOut staged) {
   constexpr int D = 128;
   constexpr int kWaveLds = 1024 + 32 * kGqaVRow;                  // P tile + V tile
   constexpr int kLoopLds = NW * kWaveLds;
@@ -347,7 +350,9 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
       l += sh_l[w * 16 + r] * cw;
       a += sh_o[(w * 16 + r) * D + d] * cw;
     }
-    out[(static_cast<size_t>(bi) * H + hk * rep + r) * D + d] = f32_to_bf16_rne(a / l);
+    const uint16_t o = f32_to_bf16_rne(a / l);
+    if (out) out[(static_cast<size_t>(bi) * H + hk * rep + r) * D + d] = o;
+    if (staged.frag) staged_store_run16(staged, bi, (hk * rep + r) * D + d, o);  // whole aligned 16-lane groups get here together
   }
 }
 
@@ -363,7 +368,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
                                                         const float *__restrict__ psum, int slices,
                                                         const uint16_t *__restrict__ col_scales,
                                                         const uint16_t *__restrict__ w, uint16_t *__restrict__ h_out,
-                                                        uint16_t *__restrict__ y, int dim, float eps) {
+                                                        uint16_t *__restrict__ y, StagedOut staged, int dim, float eps) {
   constexpr int kPieces = 2, kStride = BLOCK * 8, kWaves = BLOCK / 64;
   constexpr int kMaxSlices = 4;  // slices whose loads are all issued before the first addition
   const size_t row = blockIdx.x;
@@ -429,7 +434,9 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
     }
     return ss;
   };
-  auto scale_store = [&](u32x4_t raw, u32x4_t wr, float inv, uint16_t *dst) {
+  // y (row-major, may be null) and / or the staged form the decode-batch int4 kernels read (dim % 16 == 0 then, so the
+  // two threads that hold a run of 16 values are neighbouring lanes and take this path together)
+  auto scale_store = [&](u32x4_t raw, u32x4_t wr, float inv, int i) {
     u32x4_t o;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -437,7 +444,8 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
       const float hi = bf16_round(__builtin_bit_cast(float, raw[j] & 0xFFFF0000u) * inv) * __builtin_bit_cast(float, wr[j] & 0xFFFF0000u);
       o[j] = static_cast<uint32_t>(f32_to_bf16_rne(lo)) | (static_cast<uint32_t>(f32_to_bf16_rne(hi)) << 16);
     }
-    *reinterpret_cast<u32x4_t *>(dst) = o;
+    if (y) *reinterpret_cast<u32x4_t *>(y + row * dim + i) = o;
+    if (staged.frag) staged_store_piece(staged, static_cast<int>(row), i >> 3, o);
   };
 
   u32x4_t keep[kPieces], keepd[kPieces], keepw[kPieces];
@@ -480,14 +488,13 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const uint16_t *__restri
   for (int wv = 0; wv < kWaves; ++wv) ss += part[wv];
   const float inv = rsqrtf(ss / static_cast<float>(dim) + eps);
   const uint16_t *src = adds ? h_out + row * dim : xr;
-  uint16_t *yr = y + row * dim;
 #pragma unroll
   for (int p = 0; p < kPieces; ++p) {
     const int i = threadIdx.x * 8 + p * kStride;
-    if (i < dim) scale_store(keep[p], keepw[p], inv, yr + i);
+    if (i < dim) scale_store(keep[p], keepw[p], inv, i);
   }
   for (int i = threadIdx.x * 8 + kPieces * kStride; i < dim; i += kStride)
-    scale_store(*reinterpret_cast<const u32x4_t *>(src + i), *reinterpret_cast<const u32x4_t *>(w + i), inv, yr + i);
+    scale_store(*reinterpret_cast<const u32x4_t *>(src + i), *reinterpret_cast<const u32x4_t *>(w + i), inv, i);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -562,23 +569,23 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *__restric
 
 // few rows (decode): 512 threads so that a 4096-wide row is one piece per thread; many rows: 256-thread workgroups
 void launch_rmsnorm(const uint16_t *x, const uint16_t *delta, const float *psum, int slices, const uint16_t *col_scales, const uint16_t *w,
-                    uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps, hipStream_t stream) {
+                    uint16_t *h_out, uint16_t *y, StagedOut staged, int64_t rows, int64_t dim, float eps, hipStream_t stream) {
   if (rows <= 512 && dim >= 4096)
     hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(static_cast<unsigned>(rows)), dim3(512), 0, stream, x, delta, psum, slices, col_scales, w, h_out,
-                       y, static_cast<int>(dim), eps);
+                       y, staged, static_cast<int>(dim), eps);
   else
     hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(static_cast<unsigned>(rows)), dim3(256), 0, stream, x, delta, psum, slices, col_scales, w, h_out,
-                       y, static_cast<int>(dim), eps);
+                       y, staged, static_cast<int>(dim), eps);
 }
 
 template <int D, int NW>
 int launch_attention_nw(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
-                        const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
+                        const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale, StagedOut staged) {
   switch (rep) {
-    case 1: hipLaunchKernelGGL((decode_attention_kernel<D, 1, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
-    case 2: hipLaunchKernelGGL((decode_attention_kernel<D, 2, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
-    case 4: hipLaunchKernelGGL((decode_attention_kernel<D, 4, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
-    case 8: hipLaunchKernelGGL((decode_attention_kernel<D, 8, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale); break;
+    case 1: hipLaunchKernelGGL((decode_attention_kernel<D, 1, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale, staged); break;
+    case 2: hipLaunchKernelGGL((decode_attention_kernel<D, 2, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale, staged); break;
+    case 4: hipLaunchKernelGGL((decode_attention_kernel<D, 4, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale, staged); break;
+    case 8: hipLaunchKernelGGL((decode_attention_kernel<D, 8, NW>), grid, dim3(64 * NW), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale, staged); break;
     default: return E2H_ERR_BAD_SHAPE;
   }
   return launch_status();
@@ -588,19 +595,19 @@ int launch_attention_nw(int rep, dim3 grid, hipStream_t s, const uint16_t *q, co
 // eight waves for caches beyond 256 positions halve the tiles a wave walks through one after the other.
 template <int D>
 int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const uint16_t *kc, const uint16_t *vc, uint16_t *out,
-                     const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale) {
+                     const int64_t *input_pos, const int64_t *left_pad, int H, int Hkv, int S, float scale, StagedOut staged) {
   const int nw = options().attention_waves ? options().attention_waves : (S > 256 ? 8 : 4);
   if (D == 128 && rep >= 4 && rep <= 16 && !options().attention_no_mfma) {
     // several query heads per K / V row: both products on the matrix cores; four waves measured faster than eight
     // (three workgroups fit a CU instead of one)
     if (options().attention_waves == 8)
-      hipLaunchKernelGGL(decode_attention_gqa_kernel<8>, grid, dim3(512), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale);
+      hipLaunchKernelGGL(decode_attention_gqa_kernel<8>, grid, dim3(512), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale, staged);
     else
-      hipLaunchKernelGGL(decode_attention_gqa_kernel<4>, grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale);
+      hipLaunchKernelGGL(decode_attention_gqa_kernel<4>, grid, dim3(256), 0, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, rep, scale, staged);
     return launch_status();
   }
-  if (nw == 8) return launch_attention_nw<D, 8>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale);
-  return launch_attention_nw<D, 4>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale);
+  if (nw == 8) return launch_attention_nw<D, 8>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale, staged);
+  return launch_attention_nw<D, 4>(rep, grid, s, q, kc, vc, out, input_pos, left_pad, H, Hkv, S, scale, staged);
 }
 
 }  // namespace
@@ -608,28 +615,45 @@ int launch_attention(int rep, dim3 grid, hipStream_t s, const uint16_t *q, const
 
 using namespace e2h;
 
-extern "C" int e2h_decode_attention(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
-                                    const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch, int64_t n_head,
-                                    int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale, void *stream) {
-  if (!q || !k_cache || !v_cache || !out || !input_pos) return E2H_ERR_NULL_POINTER;
+namespace {
+int decode_attention_impl(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out, void *staged,
+                          const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch, int64_t n_head, int64_t n_kv_head,
+                          int64_t cache_len, int64_t head_dim, float scale, void *stream) {
+  if (!q || !k_cache || !v_cache || (!out && !staged) || !input_pos) return E2H_ERR_NULL_POINTER;
   if (batch < 1 || n_head < 1 || n_kv_head < 1 || n_head % n_kv_head != 0 || cache_len < 1 || batch * n_kv_head > INT32_MAX)
     return E2H_ERR_BAD_SHAPE;
-  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return E2H_ERR_MISALIGNED;
+  if (staged && (batch > 64 || (n_head * head_dim) % 128 != 0)) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(staged)) return E2H_ERR_MISALIGNED;
   const int rep = static_cast<int>(n_head / n_kv_head);
   dim3 grid(static_cast<unsigned>(batch * n_kv_head));
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const StagedOut so = staged_out(staged, batch, n_head * head_dim);
   if (head_dim == 128)
-    return launch_attention<128>(rep, grid, s, q, k_cache, v_cache, out, input_pos, left_pad_mask_pos, (int)n_head, (int)n_kv_head, (int)cache_len, scale);
+    return launch_attention<128>(rep, grid, s, q, k_cache, v_cache, out, input_pos, left_pad_mask_pos, (int)n_head, (int)n_kv_head, (int)cache_len, scale, so);
   if (head_dim == 64)
-    return launch_attention<64>(rep, grid, s, q, k_cache, v_cache, out, input_pos, left_pad_mask_pos, (int)n_head, (int)n_kv_head, (int)cache_len, scale);
+    return launch_attention<64>(rep, grid, s, q, k_cache, v_cache, out, input_pos, left_pad_mask_pos, (int)n_head, (int)n_kv_head, (int)cache_len, scale, so);
   return E2H_ERR_BAD_SHAPE;
+}
+}  // namespace
+
+extern "C" int e2h_decode_attention(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out,
+                                    const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch, int64_t n_head,
+                                    int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale, void *stream) {
+  if (!out) return E2H_ERR_NULL_POINTER;
+  return decode_attention_impl(q, k_cache, v_cache, out, nullptr, input_pos, left_pad_mask_pos, batch, n_head, n_kv_head, cache_len, head_dim, scale, stream);
+}
+
+extern "C" int e2h_decode_attention_staged(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out, void *staged,
+                                           const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch, int64_t n_head,
+                                           int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale, void *stream) {
+  return decode_attention_impl(q, k_cache, v_cache, out, staged, input_pos, left_pad_mask_pos, batch, n_head, n_kv_head, cache_len, head_dim, scale, stream);
 }
 
 extern "C" int e2h_rmsnorm(const uint16_t *x, const uint16_t *weight, uint16_t *y, int64_t rows, int64_t dim, float eps, void *stream) {
   if (!x || !weight || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, nullptr, nullptr, 0, nullptr, weight, nullptr, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, nullptr, nullptr, 0, nullptr, weight, nullptr, y, StagedOut{}, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 
@@ -638,7 +662,7 @@ extern "C" int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const u
   if (!x || !delta || !weight || !h_out || !y) return E2H_ERR_NULL_POINTER;
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(delta) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y)) return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, delta, nullptr, 0, nullptr, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, delta, nullptr, 0, nullptr, weight, h_out, y, StagedOut{}, rows, dim, eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 
@@ -649,7 +673,24 @@ extern "C" int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials
   if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX || slices < 1 || slices > 64) return E2H_ERR_BAD_SHAPE;
   if (!aligned16(x) || !aligned16(partials) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y) || (col_scales && !aligned16(col_scales)))
     return E2H_ERR_MISALIGNED;
-  launch_rmsnorm(x, nullptr, partials, slices, col_scales, weight, h_out, y, rows, dim, eps, static_cast<hipStream_t>(stream));
+  launch_rmsnorm(x, nullptr, partials, slices, col_scales, weight, h_out, y, StagedOut{}, rows, dim, eps, static_cast<hipStream_t>(stream));
+  return launch_status();
+}
+
+extern "C" int e2h_add_rmsnorm_staged(const uint16_t *x, const uint16_t *delta, const float *partials, int slices, const uint16_t *col_scales,
+                                      const uint16_t *weight, uint16_t *h_out, uint16_t *y, void *staged, int64_t rows, int64_t dim, float eps,
+                                      void *stream) {
+  if (!x || !weight || (!y && !staged)) return E2H_ERR_NULL_POINTER;
+  if (delta && partials) return E2H_ERR_BAD_SHAPE;
+  if ((delta || partials) && !h_out) return E2H_ERR_NULL_POINTER;
+  if (rows < 1 || dim < 8 || dim % 8 != 0 || rows > INT32_MAX) return E2H_ERR_BAD_SHAPE;
+  if (partials && (slices < 1 || slices > 64)) return E2H_ERR_BAD_SHAPE;
+  if (staged && (rows > 64 || dim % 128 != 0)) return E2H_ERR_BAD_SHAPE;
+  if (!aligned16(x) || !aligned16(delta) || !aligned16(partials) || !aligned16(weight) || !aligned16(h_out) || !aligned16(y) ||
+      !aligned16(staged) || !aligned16(col_scales))
+    return E2H_ERR_MISALIGNED;
+  launch_rmsnorm(x, delta, partials, partials ? slices : 0, partials ? col_scales : nullptr, weight, h_out, y, staged_out(staged, rows, dim), rows, dim,
+                 eps, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 

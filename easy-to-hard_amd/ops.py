@@ -672,3 +672,171 @@ def decode_attention(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, sca
                                           bsz, n_head, k_cache.shape[1], k_cache.shape[2], head_dim, float(scale), _stream(q))
     _lib.check(rc, "e2h_decode_attention")
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# decode batches on staged activations: the int4 kernels of csrc/e2h_int4_staged.hip read their activations in
+# matrix-core operand order, written by the kernel that produces them (norm, attention, gated feed-forward) or
+# by stage_x for activations that arrive row-major
+# ---------------------------------------------------------------------------------------------
+
+STAGED_PLAIN, STAGED_GATE, STAGED_ROPE, STAGED_PARTIAL = 0, 1, 2, 3
+
+
+class StagedActivations:
+    """`rows` x `k` bfloat16 activations in the operand order of the decode-batch int4 kernels, plus their sums over
+    runs of 16 (csrc/e2h_staged.h describes the layout).  `buf` is the flat uint8 device buffer."""
+
+    def __init__(self, buf, rows, k):
+        self.buf, self.rows, self.k = buf, rows, k
+
+    @property
+    def device(self):
+        return self.buf.device
+
+
+def staged_empty(rows, k, device):
+    nbytes = int(_lib.load().e2h_int4_staged_bytes(rows, k))
+    if nbytes <= 0:
+        raise RuntimeError(f"staged activations need 1 <= rows <= 64 and k % 128 == 0, got rows={rows}, k={k}")
+    return StagedActivations(torch.empty((nbytes,), dtype=torch.uint8, device=device), rows, k)
+
+
+def stage_x(x):
+    """x bf16 [rows <= 64, k] row-major -> StagedActivations (one pass over x)."""
+    _need_gpu(x)
+    assert x.dtype == torch.bfloat16 and x.dim() == 2
+    x = x.contiguous()
+    out = staged_empty(x.shape[0], x.shape[1], x.device)
+    rc = _lib_for(x).e2h_int4_stage_x(_ptr(x), _ptr(out.buf), x.shape[0], x.shape[1], _stream(x))
+    _lib.check(rc, "e2h_int4_stage_x")
+    return out
+
+
+def int4_staged_supported(rows, lin, epilogue):
+    """True when the staged decode-batch kernel covers `lin` (a WeightOnlyInt4Linear) at `rows` rows with the epilogue."""
+    if getattr(lin, "padding", False) or lin.inner_k_tiles != 8 or lin.weight.dim() != 4 or not lin.weight.is_cuda:
+        return False
+    if lin.scales_and_zeros.dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().e2h_int4_mm_staged_supported(rows, lin.out_features, lin.in_features, lin.groupsize, epilogue))
+
+
+def _staged_dims(xs, packed, sz, groupsize, what):
+    n, k, ikt = _packed_dims(packed)
+    if ikt != 8 or xs.k != k:
+        raise RuntimeError(f"{what}: staged activations have K={xs.k}, packed weight has K={k}, inner_k_tiles={ikt} (8 expected)")
+    if tuple(sz.shape) != (k // groupsize, n, 2) or sz.dtype != torch.bfloat16:
+        raise RuntimeError(f"{what}: scales_and_zeros must be bfloat16 [{k // groupsize}, {n}, 2], got {sz.dtype} {tuple(sz.shape)}")
+    return n, k
+
+
+def int4_mm_staged(xs, packed, groupsize, scales_and_zeros):
+    """int4_mm on staged activations -> bf16 [rows, N]."""
+    _need_gpu(xs.buf, packed, scales_and_zeros)
+    n, k = _staged_dims(xs, packed, scales_and_zeros, groupsize, "int4_mm_staged")
+    y = torch.empty((xs.rows, n), dtype=torch.bfloat16, device=xs.device)
+    rc = _lib_for(y).e2h_int4_mm_staged(_ptr(xs.buf), _ptr(packed), _ptr(scales_and_zeros), _ptr(y), xs.rows, n, k, groupsize, _stream(y))
+    _lib.check(rc, "e2h_int4_mm_staged")
+    return y
+
+
+def int4_staged_partial_slices(rows, lin):
+    s = _lib.load().e2h_int4_mm_staged_partial_slices(rows, lin.out_features, lin.in_features, lin.groupsize)
+    return s if s > 0 else 0
+
+
+def int4_mm_staged_partials(xs, packed, groupsize, scales_and_zeros, slices):
+    """-> float32 [slices, rows, N]: the sums over `slices` contiguous parts of K, for add_rmsnorm_staged to add in order."""
+    _need_gpu(xs.buf, packed, scales_and_zeros)
+    n, k = _staged_dims(xs, packed, scales_and_zeros, groupsize, "int4_mm_staged_partials")
+    out = torch.empty((slices, xs.rows, n), dtype=torch.float32, device=xs.device)
+    rc = _lib_for(out).e2h_int4_mm_staged_partials(_ptr(xs.buf), _ptr(packed), _ptr(scales_and_zeros), _ptr(out), xs.rows, n, k, groupsize,
+                                                   slices, _stream(out))
+    _lib.check(rc, "e2h_int4_mm_staged_partials")
+    return out
+
+
+def int4_mm_staged_silu_gate(xs, packed_gate, sz_gate, packed_up, sz_up, groupsize, want_rows=False, want_staged=True):
+    """bf16(bf16(silu(gate x)) * up x) for two packed weights of equal shape.  Returns (y or None, StagedActivations or None):
+    the row-major result and / or its staged form for the next linear (N % 128 == 0 then)."""
+    _need_gpu(xs.buf, packed_gate, sz_gate, packed_up, sz_up)
+    n, k = _staged_dims(xs, packed_gate, sz_gate, groupsize, "int4_mm_staged_silu_gate")
+    if _staged_dims(xs, packed_up, sz_up, groupsize, "int4_mm_staged_silu_gate") != (n, k):
+        raise RuntimeError("int4_mm_staged_silu_gate: the two packed weights differ in shape")
+    y = torch.empty((xs.rows, n), dtype=torch.bfloat16, device=xs.device) if want_rows else None
+    out = staged_empty(xs.rows, n, xs.device) if want_staged else None
+    rc = _lib_for(xs.buf).e2h_int4_mm_staged_silu_gate(_ptr(xs.buf), _ptr(packed_gate), _ptr(sz_gate), _ptr(packed_up), _ptr(sz_up),
+                                                       _ptr(y) if y is not None else None, _ptr(out.buf) if out is not None else None,
+                                                       xs.rows, n, k, groupsize, _stream(xs.buf))
+    _lib.check(rc, "e2h_int4_mm_staged_silu_gate")
+    return y, out
+
+
+def int4_mm_staged_rope_kv(xs, packed, scales_and_zeros, groupsize, freqs_cis, k_cache, v_cache, input_pos, n_head, n_kv_head, head_dim):
+    """int4_mm_rope_kv on staged activations: fused q|k|v projection, RoPE, cache write; returns the rotated q [B, H, D]."""
+    _need_gpu(xs.buf, packed, scales_and_zeros, freqs_cis, k_cache, v_cache, input_pos)
+    assert freqs_cis.dtype == torch.bfloat16 and input_pos.dtype == torch.int64 and input_pos.numel() >= 1
+    assert k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and freqs_cis.is_contiguous()
+    n, k = _staged_dims(xs, packed, scales_and_zeros, groupsize, "int4_mm_staged_rope_kv")
+    bsz = xs.rows
+    if n != (n_head + 2 * n_kv_head) * head_dim:
+        raise RuntimeError(f"int4_mm_staged_rope_kv: weight has N={n}, expected {(n_head + 2 * n_kv_head) * head_dim}")
+    if k_cache.shape[0] < bsz or k_cache.shape[1] != n_kv_head or k_cache.shape[3] != head_dim or v_cache.shape != k_cache.shape:
+        raise RuntimeError("int4_mm_staged_rope_kv: caches must be [>= B, Hkv, S, D]")
+    if freqs_cis.shape[0] < k_cache.shape[2] or tuple(freqs_cis.shape[1:]) != (head_dim // 2, 2):
+        raise RuntimeError("int4_mm_staged_rope_kv: freqs_cis must be [>= S, D/2, 2]")
+    q = torch.empty((bsz, n_head, head_dim), dtype=torch.bfloat16, device=xs.device)
+    rc = _lib_for(q).e2h_int4_mm_staged_rope_kv(_ptr(xs.buf), _ptr(packed), _ptr(scales_and_zeros), _ptr(freqs_cis), _ptr(q), _ptr(k_cache),
+                                                _ptr(v_cache), _ptr(input_pos), bsz, n_head, n_kv_head, head_dim, k_cache.shape[2], k,
+                                                groupsize, _stream(q))
+    _lib.check(rc, "e2h_int4_mm_staged_rope_kv")
+    return q
+
+
+def add_rmsnorm_staged(x, delta, weight, eps, want_rows=False):
+    """RMSNorm of h = x (delta None) or h = bf16(x + delta) (delta bf16 of x's shape, or float32 partial sums
+    [slices, rows, dim]) with the normalised rows handed on as StagedActivations.  Returns (h, y or None, staged)."""
+    _need_gpu(x, weight)
+    assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+    x = x.contiguous()
+    dim = x.shape[-1]
+    rows = x.numel() // dim
+    staged = staged_empty(rows, dim, x.device)
+    y = torch.empty_like(x) if want_rows else None
+    d16 = part = None
+    slices = 0
+    h = x
+    if delta is not None:
+        h = torch.empty_like(x)
+        if delta.dtype == torch.float32:
+            assert delta.dim() == 3 and delta.is_contiguous() and delta.shape[1] == rows and delta.shape[2] == dim
+            part, slices = delta, delta.shape[0]
+        else:
+            assert delta.dtype == torch.bfloat16 and delta.shape == x.shape
+            d16 = delta.contiguous()
+    rc = _lib_for(x).e2h_add_rmsnorm_staged(_ptr(x), _ptr(d16) if d16 is not None else None, _ptr(part) if part is not None else None, slices,
+                                            None, _ptr(weight), _ptr(h) if delta is not None else None, _ptr(y) if y is not None else None,
+                                            _ptr(staged.buf), rows, dim, float(eps), _stream(x))
+    _lib.check(rc, "e2h_add_rmsnorm_staged")
+    return h, y, staged
+
+
+def decode_attention_staged(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, scale=None):
+    """decode_attention with the result [B, H * D] handed on as StagedActivations (the input of the output projection)."""
+    _need_gpu(q, k_cache, v_cache, input_pos)
+    assert q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and input_pos.dtype == torch.int64
+    q = q.contiguous()
+    bsz, n_head, head_dim = q.shape
+    if scale is None:
+        scale = head_dim ** -0.5
+    lp = None
+    if left_pad_mask_pos is not None:
+        lp = left_pad_mask_pos.to(torch.int64).contiguous()
+    staged = staged_empty(bsz, n_head * head_dim, q.device)
+    rc = _lib_for(q).e2h_decode_attention_staged(_ptr(q), _ptr(k_cache), _ptr(v_cache), None, _ptr(staged.buf), _ptr(input_pos),
+                                                 _ptr(lp) if lp is not None else None, bsz, n_head, k_cache.shape[1], k_cache.shape[2],
+                                                 head_dim, float(scale), _stream(q))
+    _lib.check(rc, "e2h_decode_attention_staged")
+    return staged

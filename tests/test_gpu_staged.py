@@ -1,0 +1,197 @@
+"""GPU parity of the decode-batch int4 kernels that read staged activations (csrc/e2h_int4_staged.hip), through the
+C ABI: the staging pass and every producer of staged activations against a numpy restatement of the layout, the
+matmul epilogues against the float32 dequantize-then-matmul oracle (gate max|y - y_ref| / max|y_ref| <= 1e-2) and,
+bit for bit, against each other."""
+
+import numpy as np
+import pytest
+import torch
+
+from easy_to_hard_amd import ops
+from oracle import quant_oracle as qo
+from tests.helpers import bf16_to_np, randn_bf16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-2
+
+
+def _case(n, k, g, seed=1234):
+    w = randn_bf16((n, k), std=0.02, seed=seed)
+    codes, sz = qo.int4_group_quantize(bf16_to_np(w), 4, g)
+    packed = qo.int4_tile_pack(codes, 8)
+    return codes, sz, torch.from_numpy(packed).to(DEV), torch.from_numpy(sz).to(torch.bfloat16).to(DEV)
+
+
+def _staged_reference(x):
+    """numpy restatement of the staged layout for x float32 [m, k] holding bfloat16 values: (frag bits uint16
+    [k/32][mpad][32], sums float32 [k/128][mpad][8]); rows m .. mpad-1 zero."""
+    m, k = x.shape
+    mpad = (m + 15) // 16 * 16
+    bits = np.zeros((mpad, k), dtype=np.uint16)
+    bits[:m] = qo.bf16_bits(x)
+    dw = bits.reshape(mpad, k // 32, 16, 2)                     # [m][segment][dword][half]
+    pos = np.array([4 * (d % 4) + d // 4 for d in range(16)])   # original dword d -> position 4 j + i, d = j + 4 i
+    frag = np.zeros_like(dw)
+    frag[:, :, pos] = dw
+    frag = frag.transpose(1, 0, 2, 3).reshape(k // 32, mpad, 32)
+    xp = np.zeros((mpad, k), dtype=np.float32)
+    xp[:m] = x
+    v = xp.reshape(mpad, k // 16, 16)
+    for _ in range(4):                                          # balanced tree in index order, float32 at every level
+        v = (v[..., 0::2] + v[..., 1::2]).astype(np.float32)
+    sums = v.reshape(mpad, k // 128, 8).transpose(1, 0, 2)
+    return frag, sums
+
+
+def _unpack_staged(xs):
+    mpad = (xs.rows + 15) // 16 * 16
+    raw = xs.buf.cpu().numpy()
+    nfrag = mpad * xs.k * 2
+    frag = raw[:nfrag].view(np.uint16).reshape(xs.k // 32, mpad, 32)
+    sums = raw[nfrag:].view(np.float32).reshape(xs.k // 128, mpad, 8)
+    return frag, sums
+
+
+def _assert_staged_equal(xs, x_np, rows):
+    frag, sums = _unpack_staged(xs)
+    frag_ref, sums_ref = _staged_reference(x_np)
+    assert np.array_equal(frag[:, :rows], frag_ref[:, :rows])
+    assert np.array_equal(sums[:, :rows].view(np.uint32), sums_ref[:, :rows].view(np.uint32))
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 33, 64])
+def test_stage_x_layout_and_sums(m):
+    k = 512
+    x = randn_bf16((m, k), seed=m)
+    xs = ops.stage_x(x.to(DEV))
+    assert xs.rows == m and xs.k == k
+    _assert_staged_equal(xs, bf16_to_np(x), m)
+    frag, sums = _unpack_staged(xs)
+    assert not frag[:, m:].any() and not sums[:, m:].any()  # padding rows are written as zeros by this pass
+
+
+@pytest.mark.parametrize("g", [32, 64, 128])
+@pytest.mark.parametrize("shape", [(48, 512), (64, 1024), (4096, 4096), (1024, 11008)])
+def test_staged_mm_plain_and_partials_against_the_oracle(g, shape):
+    n, k = shape
+    codes, sz, packed_d, sz_d = _case(n, k, g, seed=g + n)
+    for m in (1, 16, 17, 32, 33, 64):
+        x = randn_bf16((m, k), seed=m)
+        xs = ops.stage_x(x.to(DEV))
+        y_ref = qo.int4_linear_fp32(bf16_to_np(x), codes, sz, g)
+        lin = _Lin(n, k, g, packed_d, sz_d)
+        if ops.int4_staged_supported(m, lin, ops.STAGED_PLAIN):
+            y = ops.int4_mm_staged(xs, packed_d, g, sz_d)
+            assert qo.normwise_rel_err(bf16_to_np(y), y_ref) <= TOL
+            assert qo.elementwise_violations(bf16_to_np(y), y_ref) == 0.0
+        assert ops.int4_staged_supported(m, lin, ops.STAGED_PARTIAL), (m, n, k, g)
+        s = ops.int4_staged_partial_slices(m, lin)
+        assert s >= 1
+        part = ops.int4_mm_staged_partials(xs, packed_d, g, sz_d, s)
+        assert part.shape == (s, m, n) and part.dtype == torch.float32
+        total = part[0].clone()
+        for i in range(1, s):
+            total += part[i]  # slice order, float32: what the consumer adds
+        yp = total.to(torch.bfloat16)
+        assert qo.normwise_rel_err(bf16_to_np(yp), y_ref) <= TOL
+        again = ops.int4_mm_staged_partials(xs, packed_d, g, sz_d, s)
+        assert torch.equal(part, again)  # fixed summation order: run to run bit equality
+
+
+class _Lin:
+    """The attributes of a WeightOnlyInt4Linear the support queries read."""
+
+    def __init__(self, n, k, g, packed, sz):
+        self.out_features, self.in_features, self.groupsize, self.inner_k_tiles = n, k, g, 8
+        self.weight, self.scales_and_zeros, self.padding = packed, sz, False
+
+
+def test_staged_mm_exact_small_integers():
+    # activations and dequantized weights are small integers: every product and sum is exact, so the result must equal
+    # the integer matmul exactly
+    n, k, g = 64, 512, 128
+    rng = np.random.default_rng(3)
+    codes = rng.integers(0, 16, size=(n, k)).astype(np.int32)
+    sz = np.zeros((k // g, n, 2), dtype=np.float32)
+    sz[..., 0] = 1.0   # scale 1
+    sz[..., 1] = 8.0   # zero 8: w = q
+    packed_d = torch.from_numpy(qo.int4_tile_pack(codes, 8)).to(DEV)
+    sz_d = torch.from_numpy(sz).to(torch.bfloat16).to(DEV)
+    x = torch.from_numpy(rng.integers(-2, 3, size=(32, k)).astype(np.float32)).to(torch.bfloat16)
+    xs = ops.stage_x(x.to(DEV))
+    s = ops.int4_staged_partial_slices(32, _Lin(n, k, g, packed_d, sz_d))
+    part = ops.int4_mm_staged_partials(xs, packed_d, g, sz_d, s).sum(0)
+    want = bf16_to_np(x).astype(np.int64) @ codes.T.astype(np.int64)
+    assert np.array_equal(part.cpu().numpy().astype(np.int64), want)
+
+
+@pytest.mark.parametrize("g", [64, 128])
+def test_staged_gate_equals_the_unfused_staged_calls_and_hands_on_staged_rows(g):
+    n, k = 1536, 4096   # n % 128 == 0: the result is the next linear's K
+    _, _, pg, szg = _case(n, k, g, seed=11)
+    _, _, pu, szu = _case(n, k, g, seed=12)
+    for m in (8, 32, 48):
+        x = randn_bf16((m, k), seed=m)
+        xs = ops.stage_x(x.to(DEV))
+        lin = _Lin(n, k, g, pg, szg)
+        assert ops.int4_staged_supported(m, lin, ops.STAGED_GATE)
+        y, ys = ops.int4_mm_staged_silu_gate(xs, pg, szg, pu, szu, g, want_rows=True, want_staged=True)
+        # the plain epilogue splits K the same way, so the fused result must equal the unfused calls bit for bit
+        assert ops.int4_staged_supported(m, lin, ops.STAGED_PLAIN)
+        a = ops.int4_mm_staged(xs, pg, g, szg)
+        b = ops.int4_mm_staged(xs, pu, g, szu)
+        assert torch.equal(y, ops.silu_mul(a, b))
+        _assert_staged_equal(ys, bf16_to_np(y), m)
+
+
+def test_staged_rope_kv_equals_projection_then_rope_kernel():
+    n_head, n_kv, hd, k, g, s_max, bsz = 8, 2, 128, 1024, 128, 64, 32
+    n = (n_head + 2 * n_kv) * hd
+    _, _, packed_d, sz_d = _case(n, k, g, seed=5)
+    from easy_to_hard_amd.model import precompute_freqs_cis
+
+    freqs = precompute_freqs_cis(s_max, hd, 10000, device=DEV)
+    x = randn_bf16((bsz, k), seed=9).to(DEV)
+    xs = ops.stage_x(x)
+    pos = torch.tensor([17], dtype=torch.int64, device=DEV)
+    kc = torch.zeros((bsz, n_kv, s_max, hd), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    assert ops.int4_staged_supported(bsz, _Lin(n, k, g, packed_d, sz_d), ops.STAGED_ROPE)
+    q = ops.int4_mm_staged_rope_kv(xs, packed_d, sz_d, g, freqs, kc, vc, pos, n_head, n_kv, hd)
+    qkv = ops.int4_mm_staged(xs, packed_d, g, sz_d)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2 = ops.rope_kv_write(qkv, freqs, kc2, vc2, pos, n_head, n_kv, hd)
+    assert torch.equal(q, q2) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 512), (32, 4096), (33, 1024), (64, 8192)])
+def test_add_rmsnorm_staged_equals_the_row_major_kernel(rows, dim):
+    x = randn_bf16((rows, dim), seed=1).to(DEV)
+    d = randn_bf16((rows, dim), seed=2).to(DEV)
+    w = (1.0 + 0.1 * randn_bf16((dim,), seed=3).float()).to(torch.bfloat16).to(DEV)
+    part = torch.randn((3, rows, dim), generator=torch.Generator().manual_seed(4)).to(DEV)
+    y0 = ops.rmsnorm(x, w, 1e-5)
+    h, y, xs = ops.add_rmsnorm_staged(x, None, w, 1e-5, want_rows=True)
+    assert h is x and torch.equal(y, y0)
+    _assert_staged_equal(xs, bf16_to_np(y0), rows)
+    h1, y1 = ops.add_rmsnorm(x, d, w, 1e-5)
+    h, y, xs = ops.add_rmsnorm_staged(x, d, w, 1e-5)
+    assert y is None and torch.equal(h, h1)
+    _assert_staged_equal(xs, bf16_to_np(y1), rows)
+    h2, y2 = ops.add_rmsnorm(x, part, w, 1e-5)
+    h, _, xs = ops.add_rmsnorm_staged(x, part, w, 1e-5)
+    assert torch.equal(h, h2)
+    _assert_staged_equal(xs, bf16_to_np(y2), rows)
+
+
+@pytest.mark.parametrize("n_head,n_kv", [(4, 4), (8, 2), (8, 1)])
+def test_decode_attention_staged_equals_the_row_major_kernel(n_head, n_kv):
+    bsz, hd, s_max = 32, 128, 300
+    q = randn_bf16((bsz, n_head, hd), seed=1).to(DEV)
+    kc = randn_bf16((bsz, n_kv, s_max, hd), seed=2).to(DEV)
+    vc = randn_bf16((bsz, n_kv, s_max, hd), seed=3).to(DEV)
+    pos = torch.tensor([257], dtype=torch.int64, device=DEV)
+    out = ops.decode_attention(q, kc, vc, pos)
+    xs = ops.decode_attention_staged(q, kc, vc, pos)
+    _assert_staged_equal(xs, bf16_to_np(out.view(bsz, n_head * hd)), bsz)
