@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # `bench.py --gemv-only`, scaled by a 256 MiB copy; the summary with the commands is in
 # profiles/int4_skinny_mm_7b_decode_bs32.md.  Counters cannot be read from inside this process, so the figure is
 # recorded here for the configuration it was measured on and reported as null for any other.
-MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32): 33_440_000}
+MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32, "int4_skinny_mm_kernel"): 33_440_000}
 
 
 def parse_args():
@@ -48,6 +48,9 @@ def parse_args():
     ap.add_argument("--prompt", type=int, default=256)
     ap.add_argument("--max-new", type=int, default=512)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed-on", default="auto", choices=["auto", "cpu", "device"],
+                    help="where the random weights are drawn: a CPU generator with seed 1234 (identical values on every machine; "
+                         "about 8 s per billion parameters) or the GPU's generator; auto = cpu up to 8 billion parameters")
     ap.add_argument("--gemv-reps", type=int, default=20)
     ap.add_argument("--reward", action="store_true",
                     help="reward-model scoring workload instead of decode: one fully causal pass over --batch x --prompt "
@@ -63,12 +66,16 @@ def parse_args():
                          "linear goes through PyTorch-ROCm's aten._weight_int4pack_mm and everything around the linears through "
                          "stock torch ops (what the reference's model code executes, without inductor); prints its own JSON line")
     ap.add_argument("--model-switch", action="append", default=[], metavar="NAME=0|1",
-                    help="set a fusion switch of easy_to_hard_amd.model (FUSE_GATE, FUSE_ROPE_PROJECTION, DEFER_SPLIT_K) for a comparison run")
+                    help="set a fusion switch of easy_to_hard_amd.model (FUSE_GATE, FUSE_ROPE_PROJECTION, DEFER_SPLIT_K, STAGED_DECODE, STAGED_HEAD) for a comparison run")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch-geometry override passed to e2h_set_option (experiments)")
     ap.add_argument("--full-decode", action="store_true",
                     help="run the whole decode of the configuration (every position once) and print its tok/s, as a check of "
                          "the default mode's evenly spread sample of positions")
+    ap.add_argument("--floor", action="store_true",
+                    help="launch floor of this machine for the step's dequant-GEMV launches: a kernel of the library that only reads "
+                         "(e2h_stream_read_probe) is launched once per quantized-linear launch of a decode step on as many bytes as that "
+                         "launch has to read, from a HIP graph over a rotating region; prints the time per launch size and their sum")
     ap.add_argument("--gemv-only", action="store_true",
                     help="only the back-to-back dequant-GEMV pass plus a 256 MiB calibration copy (for counter runs)")
     return ap.parse_args()
@@ -99,7 +106,9 @@ def algorithmic_bytes(mod, m):
 
 
 def measure_gemv_roofline(model, batch, reps, traffic_key=None):
-    """All quantized-linear launches of one decode step, back to back from one HIP graph."""
+    """All quantized-linear launches of one decode step, back to back from one HIP graph: the same kernel instantiations
+    and epilogues the decode step runs (for an int4 model the staged decode-batch kernels with the RoPE + cache write,
+    gated and K-slice epilogues), each launch on its own layer's weights."""
     import torch
 
     dev = torch.device("cuda", 0)
@@ -109,12 +118,41 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
         if mod.in_features not in xs:
             xs[mod.in_features] = torch.randn((batch, mod.in_features), device=dev, dtype=torch.float32).to(torch.bfloat16)
 
-    # the launches of a decode step: a feed-forward block's w1 and w3 go out as one gated launch where the
-    # model does so too; every other quantized linear is one launch
     from easy_to_hard_amd import model as e2h_model
     from easy_to_hard_amd import ops
 
     calls, by_name, bytes_pass = [], dict(lins), 0
+    kernel_set = None
+    if not model.kv_cache_enabled:
+        model.setup_caches(batch, 768)
+    if model.staged_step_supported(batch):
+        kernel_set = "int4_staged_mm_kernel"
+        staged = {k: ops.stage_x(v) for k, v in xs.items()}
+        pos = torch.tensor([model.max_seq_length // 2], device=dev, dtype=torch.int64)
+        for blk in model.layers:
+            att, ff = blk.attention, blk.feed_forward
+            w, wo, w1, w3, w2 = att.wqkv, att.wo, ff.w1, ff.w3, ff.w2
+            calls.append(lambda a=att, w=w, s=staged[w.in_features]: ops.int4_mm_staged_rope_kv(
+                s, w.weight, w.scales_and_zeros, w.groupsize, a.freqs_table, a.kv_cache.k_cache, a.kv_cache.v_cache, pos, a.n_head,
+                a.n_local_heads, a.head_dim))
+            calls.append(lambda l=wo, s=staged[wo.in_features], n=ops.int4_staged_partial_slices(batch, wo): ops.int4_mm_staged_partials(
+                s, l.weight, l.groupsize, l.scales_and_zeros, n))
+            calls.append(lambda g=w1, u=w3, s=staged[w1.in_features]: ops.int4_mm_staged_silu_gate(
+                s, g.weight, g.scales_and_zeros, u.weight, u.scales_and_zeros, g.groupsize))
+            calls.append(lambda l=w2, s=staged[w2.in_features], n=ops.int4_staged_partial_slices(batch, w2): ops.int4_mm_staged_partials(
+                s, l.weight, l.groupsize, l.scales_and_zeros, n))
+            bytes_pass += algorithmic_bytes(w, batch) + algorithmic_bytes(wo, batch) + algorithmic_bytes(w2, batch)
+            # two weight matrices, but x is read once and one [batch, n] result is written
+            bytes_pass += algorithmic_bytes(w1, batch) + algorithmic_bytes(w3, batch) - batch * 2 * (w1.in_features + w1.out_features)
+        out = model.output
+        if e2h_model.STAGED_HEAD and ops.int4_staged_supported(batch, out, ops.STAGED_PLAIN):
+            calls.append(lambda l=out, s=staged[out.in_features]: ops.int4_mm_staged(s, l.weight, l.groupsize, l.scales_and_zeros))
+        else:
+            calls.append(lambda l=out, x=xs[out.in_features]: l(x))
+        bytes_pass += algorithmic_bytes(out, batch)
+        lins = []
+    # otherwise the launches of the row-major path: a feed-forward block's w1 and w3 go out as one gated launch where the
+    # model does so too; every other quantized linear is one launch
     for name, mod in lins:
         parent_name, _, leaf = name.rpartition(".")
         parent = model.get_submodule(parent_name) if parent_name else model
@@ -135,6 +173,8 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
         else:
             calls.append(lambda x=x, m=mod: m(x))
             bytes_pass += algorithmic_bytes(mod, batch)
+    if kernel_set is None:
+        kernel_set = "int4_skinny_mm_kernel" if "Int4" in type(by_name[next(iter(by_name))]).__name__ else "int8_stream_mm_kernel"
 
     def one_pass():
         out = None
@@ -169,13 +209,76 @@ def measure_gemv_roofline(model, batch, reps, traffic_key=None):
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(traffic_key),
-        "kernel": "int4_skinny_mm_kernel" if "Int4" in type(lins[0][1]).__name__ else "int8_stream_mm_kernel",
+        "traffic": MEASURED_TRAFFIC_BYTES.get(tuple(traffic_key or ()) + (kernel_set,)),
+        "kernel": kernel_set,
         "launches_per_step": len(calls),
         "algorithmic_bytes_per_launch": bytes_pass // len(calls),
         "avg_launch_us": round(avg_launch_s * 1e6, 3),
         "gemv_ms_per_step": round(total_s / reps * 1e3, 4),
     }
+
+
+def measure_launch_floor(model, batch, reps):
+    """What the step's quantized-linear launches would cost if each did nothing but read its weights and qparams: the
+    library's streaming-read kernel on the same byte counts, one launch per linear launch, replayed from a HIP graph.
+    The read regions rotate through a buffer larger than every cache."""
+    import ctypes
+
+    import torch
+
+    from easy_to_hard_amd import _lib
+
+    dev = torch.device("cuda", 0)
+    lib = _lib.load()
+    sizes = []  # weight + qparam bytes of every launch of a step (w1 and w3 share a launch)
+    for blk in model.layers:
+        att, ff = blk.attention, blk.feed_forward
+        wb = lambda m: algorithmic_bytes(m, 0)
+        sizes += [("wqkv", wb(att.wqkv)), ("wo", wb(att.wo)), ("w1+w3", wb(ff.w1) + wb(ff.w3)), ("w2", wb(ff.w2))]
+    sizes.append(("output", algorithmic_bytes(model.output, 0)))
+    region = torch.empty(3 << 30, dtype=torch.uint8, device=dev).fill_(3)
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def timed(launches):
+        """launches: list of byte counts; returns the average microseconds per launch"""
+        def one_pass():
+            off = 0
+            for nbytes in launches:
+                nbytes -= nbytes % 16
+                if off + nbytes > region.numel():
+                    off = 0
+                rc = lib.e2h_stream_read_probe(ctypes.c_void_p(region.data_ptr() + off), nbytes, None, stream())
+                assert rc == 0, rc
+                off += (nbytes + 4095) // 4096 * 4096
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            one_pass()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            one_pass()
+        graph.replay()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e3 / (reps * len(launches))
+
+    per_size = {}
+    for name, nbytes in sizes:
+        if name not in per_size:
+            per_size[name] = {"bytes": nbytes, "us": round(timed([nbytes] * 64), 2)}
+    empty_us = round(timed([0] * 256), 2)
+    step_us = timed([b for _, b in sizes]) * len(sizes)
+    total_bytes = sum(b for _, b in sizes)
+    return {"empty_launch_us": empty_us, "per_launch": per_size, "launches_per_step": len(sizes),
+            "read_only_ms_per_step": round(step_us * 1e-3, 4), "weight_bytes_per_step": total_bytes,
+            "hbm_frac_of_a_read_only_step": round(total_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "note": "a launch-per-linear decode step cannot spend less time in its quantized linears than read_only_ms_per_step"}
 
 
 def stock_int4_operands(mod):
@@ -342,7 +445,8 @@ def run_reward_scoring(args, cfg, dev):
     from easy_to_hard_amd.generate import model_score
     from easy_to_hard_amd.model import random_quantized_transformer
 
-    model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234, reward_head_rows=2)
+    model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234, reward_head_rows=2,
+                                         seed_on="device" if args.seed_on == "device" else "cpu")
     batch, t = args.batch, args.prompt
     ids = torch.randint(0, cfg.vocab_size, (batch, t), generator=torch.Generator().manual_seed(1234)).to(dev)
     steps, warmup = min(args.steps, 8), min(args.warmup, 2)
@@ -390,7 +494,7 @@ def main():
         import easy_to_hard_amd.model as model_mod
 
         name, _, value = item.partition("=")
-        assert name in ("FUSE_GATE", "FUSE_ROPE_PROJECTION", "DEFER_SPLIT_K"), name
+        assert name in ("FUSE_GATE", "FUSE_ROPE_PROJECTION", "DEFER_SPLIT_K", "STAGED_DECODE", "STAGED_HEAD"), name
         setattr(model_mod, name, bool(int(value)))
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda", 0)
@@ -404,7 +508,10 @@ def main():
         run_reward_scoring(args, cfg, dev)
         return
     t0 = time.time()
-    model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234)
+    n_params = cfg.n_layer * (cfg.dim * (cfg.n_head + 2 * cfg.n_local_heads) * cfg.head_dim + cfg.dim * cfg.dim
+                              + 3 * cfg.dim * cfg.intermediate_size) + 2 * cfg.vocab_size * cfg.dim
+    seed_on = args.seed_on if args.seed_on != "auto" else ("cpu" if n_params <= 8e9 else "device")
+    model = random_quantized_transformer(cfg, args.mode, args.groupsize, device=dev, seed=1234, seed_on=seed_on)
     torch.cuda.synchronize()
     build_s = time.time() - t0
 
@@ -420,6 +527,10 @@ def main():
                              "64 timed fully, larger ones on 512 rows and scaled (see cpu_rows_timed)"}
         print(json.dumps({"per_shape": rows_out, "model": args.model, "mode": args.mode,
                           "groupsize": args.groupsize if args.mode == "int4" else None, "cpu_baseline": cpu}))
+        return
+    if args.floor:
+        print(json.dumps({"floor": measure_launch_floor(model, batch, args.gemv_reps), "model": args.model, "mode": args.mode,
+                          "groupsize": args.groupsize if args.mode == "int4" else None, "batch": batch}))
         return
     if args.gemv_only:
         # counter-collection mode: the GEMV pass and a plain copy of known size (its FETCH_SIZE / WRITE_SIZE
@@ -535,6 +646,7 @@ def main():
             "timed_positions": f"{steps} steps at cache positions {positions[0]} .. {positions[-1]}, evenly spread over the decode",
             "step_ms_first_mid_last": [round(step_ms[0], 4), round(step_ms[steps // 2], 4), round(step_ms[-1], 4)],
             "quantized_linears_per_step": roofline["launches_per_step"],
+            "weights_seeded_on": seed_on,
             "model_build_s": round(build_s, 2),
             "prefill_s": round(prefill_s, 3),
         },

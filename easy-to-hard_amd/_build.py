@@ -15,7 +15,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_NAME = "libe2h_quant.so"
 LIB_PATH = PKG_DIR / LIB_NAME
 
-SOURCES = ["e2h_abi.hip", "e2h_quantize.hip", "e2h_int4_mm.hip", "e2h_int4_staged.hip", "e2h_int8_mm.hip", "e2h_int8_stream.hip", "e2h_int4_gemm.hip", "e2h_int4_gemm128.hip", "e2h_int8_gemm.hip", "e2h_attention.hip", "e2h_sample.hip"]
+SOURCES = ["e2h_abi.hip", "e2h_quantize.hip", "e2h_int4_mm.hip", "e2h_int4_staged.hip", "e2h_int8_mm.hip", "e2h_int8_stream.hip", "e2h_int4_gemm.hip", "e2h_int4_gemm128.hip", "e2h_int8_gemm.hip", "e2h_attention.hip", "e2h_sample.hip", "e2h_probe.hip"]
 
 # -ffp-contract=off: the quantizers are bit-exact restatements of separate torch ops; an FMA formed
 # across two of them would change codes.  packed-fp32-ops is switched off because some packed float32

@@ -3,9 +3,11 @@
 // Same contract and data layouts as e2h_int4_mm.hip (torch.ops.aten._weight_int4pack_mm as called by
 // linear_forward_int4, reference models/quantize.py:445-453), inner_k_tiles = 8, group size 32 / 64 / 128.
 //
-// Dequantize-to-bfloat16 form: every weight becomes  w = bf16( s * (q - 8) + z )  (one float32 FMA on 128 + q with the
-// constant z - 136 s, rounded to nearest even) on its way into the matrix cores, and the products accumulate in
-// float32 -- the arithmetic of the kernel the reference calls.  With 256 accumulator registers per lane there is no
+// Dequantize-to-bfloat16 form: every weight becomes a bfloat16 value w = bf16( fma(128 + q, s, fma(-136, s, z)) ) on its
+// way into the matrix cores (two float32 FMAs: the constant z - 136 s is rounded to float32 once per group, then one FMA
+// per weight, then round to nearest even; within one bfloat16 ulp of the single-rounded bf16(s * (q - 8) + z) and equal
+// to it whenever z - 136 s is exact in float32), and the products accumulate in float32 -- the arithmetic of the
+// kernel the reference calls, up to that ulp.  With 256 accumulator registers per lane there is no
 // room for per-group partial sums, and none are needed this way: no pass over x for group sums, no accumulator
 // prologue, no scaling of accumulators inside the loop.
 //

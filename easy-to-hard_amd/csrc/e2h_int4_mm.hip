@@ -771,16 +771,13 @@ int int4_mm_impl(const uint16_t *x, const int32_t *packed, const uint16_t *scale
   int64_t max_rows = rows_by_bytes < rows_by_grid ? rows_by_bytes : rows_by_grid;
   max_rows -= max_rows % (16 * mt);
   if (max_rows < 16 * mt) return E2H_ERR_BAD_SHAPE;
-  // 256 x 256 outputs per workgroup (dequantize-to-bfloat16 kernel, no group sums of x) or 128 x 256 (32x32-tile kernel
-  // with group sums from a pre-pass): a 256-row workgroup takes about 1.8 x as long as a 128-row one, so it wins when it
-  // needs fewer than 1 / 1.8 as many rounds of workgroups over the chip's CUs
-  const auto takes_256_row_kernel = [&](int64_t rows) {
-    if (!(mt == 4 && wide_ok && !options().int4_no_gemm32 && a.K % 256 == 0)) return false;
-    const long long wgs256 = static_cast<long long>((rows + 255) / 256) * ((a.N + 255) / 256);
-    const long long wgs128 = static_cast<long long>((rows + 127) / 128) * ((a.N + 255) / 256);
-    const long long rounds256 = (wgs256 + kCUs - 1) / kCUs, rounds128 = (wgs128 + kCUs - 1) / kCUs;
-    const bool enough = options().int4_gemm32_min_rows > 0 ? rows >= options().int4_gemm32_min_rows : wgs128 >= 320;
-    return options().int4_gemm_tile ? options().int4_gemm_tile == 256 : (enough && rounds256 * 20 <= rounds128 * 11);
+  // Many rows run on the 128-row kernel (exact products, scale and zero applied to float32 group sums: the arithmetic of
+  // every other int4 kernel here, so a row's result does not depend on how many rows share the call).  The 256 x 256
+  // kernel that dequantizes to bfloat16 on the way into the matrix cores (the reference kernel's arithmetic, 15-20 %
+  // faster at thousands of rows) is taken only on request, option "int4_gemm_tile" = 256, and then for every slice of
+  // the call alike.
+  const auto takes_256_row_kernel = [&](int64_t) {
+    return mt == 4 && wide_ok && !options().int4_no_gemm32 && a.K % 256 == 0 && options().int4_gemm_tile == 256;
   };
   if (mt == 4 && wide_ok && workspace && !options().int4_no_xsum && !takes_256_row_kernel(a.M)) {
     // many rows: the pre-pass keeps (K / g) sums per row in the workspace; slice M so that they fit rather than fall
@@ -856,6 +853,7 @@ extern "C" int64_t e2h_int4_mm_static_scratch_bytes(void) { return static_cast<i
 extern "C" int e2h_int4_mm_static_scratch(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
                                           int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *stream) {
   using namespace e2h;
+  if (!x || !packed || !scales_and_zeros || !y) return E2H_ERR_NULL_POINTER;
   if (m > 64) return E2H_ERR_SCRATCH_TOO_SMALL;  // larger batches keep per-row group sums in scratch: outside the fixed budget
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return E2H_ERR_NO_DEVICE;

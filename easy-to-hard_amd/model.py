@@ -3,8 +3,10 @@
 It reproduces the forward semantics and the state-dict key names of the reference's models/model.py
 (Transformer :132-252, TransformerBlock :255-283, Attention :286-349, FeedForward :352-360, RMSNorm
 :363-386, RoPE cache :389-412, KVCache :112-129, configs :78-109) so that a QuantHandler from
-quantize.py can swap its nn.Linear children and a reference checkpoint loads key for key.  Attention,
-normalisation and RoPE are stock PyTorch ops; only the linears are this package's kernels.
+quantize.py can swap its nn.Linear children and a reference checkpoint loads key for key.  On the GPU with
+bfloat16 tensors the single-token decode step runs entirely on this package's kernels (quantized linears, RMSNorm with
+the residual add, RoPE + cache write, decode attention, SiLU gate); other passes use them where a fused form exists and
+stock PyTorch ops elsewhere.
 """
 
 from dataclasses import dataclass
@@ -25,6 +27,9 @@ FUSED_DECODE = True
 FUSE_GATE = True            # silu(w1 x) * w3 x as one int4 launch
 FUSE_ROPE_PROJECTION = True  # q|k|v projection + RoPE + cache write as one int4 launch
 DEFER_SPLIT_K = True         # wo / w2 hand float32 K-slice sums to the residual add + RMSNorm instead of combining them
+STAGED_DECODE = True         # int4 decode step: activations travel between the kernels in matrix-core operand order
+STAGED_HEAD = True           # ... including the LM head
+STAGED_MAX_ROWS = 32         # beyond one 32-row slab the row-major kernels are as fast or faster (34B shapes at 64 rows)
 
 
 def _fusable(t: Tensor) -> bool:
@@ -314,6 +319,37 @@ class TransformerBlock(nn.Module):
         return h, self.feed_forward(normed2, defer_output=DEFER_SPLIT_K)
 
 
+def _staged_block_supported(blk: "TransformerBlock", rows: int) -> bool:
+    """True when every linear of the block has a decode-batch kernel on staged activations for `rows` rows."""
+    att, ff = blk.attention, blk.feed_forward
+    lins = (att.wqkv, att.wo, ff.w1, ff.w3, ff.w2)
+    if not all(isinstance(m, WeightOnlyInt4Linear) for m in lins):
+        return False
+    if ff.w1.groupsize != ff.w3.groupsize or ff.w1.weight.shape != ff.w3.weight.shape or ff.w1.out_features % 128 != 0:
+        return False
+    return (ops.int4_staged_supported(rows, att.wqkv, ops.STAGED_ROPE) and ops.int4_staged_supported(rows, att.wo, ops.STAGED_PARTIAL)
+            and ops.int4_staged_supported(rows, ff.w1, ops.STAGED_GATE) and ops.int4_staged_supported(rows, ff.w2, ops.STAGED_PARTIAL))
+
+
+def _staged_block_forward(blk: "TransformerBlock", x: Tensor, delta, input_pos: Tensor):
+    """One decoder block of the single-token step on staged activations (reference models/model.py:279-283 with
+    Attention.forward :310-349 and FeedForward.forward :359-360).  `delta` is what the previous block left to be added to
+    the residual stream (float32 K-slice sums of its w2, or None); returns (residual stream, this block's w2 sums)."""
+    att, ff = blk.attention, blk.feed_forward
+    rows = x.shape[0]
+    h, _, xs = ops.add_rmsnorm_staged(x, delta, blk.attention_norm.weight, blk.attention_norm.eps)
+    w = att.wqkv
+    q = ops.int4_mm_staged_rope_kv(xs, w.weight, w.scales_and_zeros, w.groupsize, att.freqs_table, att.kv_cache.k_cache,
+                                   att.kv_cache.v_cache, input_pos, att.n_head, att.n_local_heads, att.head_dim)
+    ys = ops.decode_attention_staged(q, att.kv_cache.k_cache, att.kv_cache.v_cache, input_pos, att.left_pad_mask_pos)
+    wo = att.wo
+    attn = ops.int4_mm_staged_partials(ys, wo.weight, wo.groupsize, wo.scales_and_zeros, ops.int4_staged_partial_slices(rows, wo))
+    h, _, xs2 = ops.add_rmsnorm_staged(h, attn, blk.ffn_norm.weight, blk.ffn_norm.eps)
+    _, gs = ops.int4_mm_staged_silu_gate(xs2, ff.w1.weight, ff.w1.scales_and_zeros, ff.w3.weight, ff.w3.scales_and_zeros, ff.w1.groupsize)
+    w2 = ff.w2
+    return h, ops.int4_mm_staged_partials(gs, w2.weight, w2.groupsize, w2.scales_and_zeros, ops.int4_staged_partial_slices(rows, w2))
+
+
 class Transformer(nn.Module):
     def __init__(self, config: ModelArgs) -> None:
         super().__init__()
@@ -354,6 +390,20 @@ class Transformer(nn.Module):
         self.causal_mask = torch.tril(torch.ones(max_seq_length, max_seq_length, dtype=torch.bool, device=device))
         self.self_mask = torch.eye(max_seq_length, dtype=torch.bool, device=device)
 
+    def staged_step_supported(self, rows: int) -> bool:
+        """True when a single-token step of `rows` sequences runs on the decode-batch int4 kernels with staged activations
+        (an int4 model on the GPU with bfloat16 norms and caches set up, at most STAGED_MAX_ROWS sequences)."""
+        if not (FUSED_DECODE and STAGED_DECODE and FUSE_GATE and FUSE_ROPE_PROJECTION and DEFER_SPLIT_K) or torch.compiler.is_compiling():
+            return False
+        if not (1 <= rows <= STAGED_MAX_ROWS and self.config.dim % 128 == 0 and self.kv_cache_enabled and self.freqs_cis is not None):
+            return False
+        if self.norm.weight.dtype != torch.bfloat16 or not self.norm.weight.is_cuda or self.freqs_cis.dtype != torch.bfloat16:
+            return False
+        att = self.layers[0].attention
+        if att.kv_cache is None or self.freqs_cis.shape[0] < att.kv_cache.k_cache.shape[2]:
+            return False
+        return all(_staged_block_supported(blk, rows) for blk in self.layers)
+
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None, left_pad_mask_pos: Optional[Tensor] = None,
                 fully_causal: bool = False) -> Tensor:
         """idx [B, S] token ids, input_pos [S] positions -> logits [B, S, vocab] (reference :212-248)."""
@@ -374,6 +424,18 @@ class Transformer(nn.Module):
         if fused_step and input_pos.dtype != torch.int64:
             # the reference decodes with an int32 position tensor (inference_generate.py:205); the fused kernels read int64
             input_pos = input_pos.to(torch.int64)
+        if fused_step and self.staged_step_supported(x.shape[0]):
+            # single-token step of an int4 model: every activation between two kernels travels in operand order
+            rows = x.shape[0]
+            h, delta = x.view(rows, -1), None
+            for blk in self.layers:
+                h, delta = _staged_block_forward(blk, h, delta, input_pos)
+            out = self.output
+            if isinstance(out, WeightOnlyInt4Linear) and STAGED_HEAD and ops.int4_staged_supported(rows, out, ops.STAGED_PLAIN):
+                _, _, xs = ops.add_rmsnorm_staged(h, delta, self.norm.weight, self.norm.eps)
+                return ops.int4_mm_staged(xs, out.weight, out.groupsize, out.scales_and_zeros).view(rows, 1, -1)
+            _, normed = ops.add_rmsnorm(h, delta, self.norm.weight, self.norm.eps)
+            return self.output(normed.view(rows, 1, -1))
         if _fusable(x) and x.shape[-1] % 8 == 0 and self.norm.weight.dtype == torch.bfloat16:
             delta = None
             for layer in self.layers:
@@ -411,12 +473,18 @@ class RewardModel(nn.Module):
         return cls(ModelArgs.from_name(name), head_rows)
 
 
-def apply_reward_modeling_head(transformer: "Transformer", requires_grad: bool = False, init_scheme: str = "zeros") -> None:
+def apply_reward_modeling_head(transformer: "Transformer", requires_grad: bool = False, init_scheme: Optional[str] = None,
+                               init_sceheme: Optional[str] = None) -> None:
     """Turn a language model's `output` projection into the two-row score head, in place (reference
-    models/reward_model.py:95-133): "zeros" starts from a zero head, "semantic" from the rows of the tokens "2" (id 29906)
-    and, negated, "1" (id 29896) of the existing projection, "random" from a Kaiming-uniform draw (seed 42) scaled by
-    sqrt(2).  The head keeps the dtype and device of the projection it replaces."""
+    models/reward_model.py:95-133): "zeros" (the default) starts from a zero head, "semantic" from the rows of the tokens
+    "2" (id 29906) and, negated, "1" (id 29896) of the existing projection, "random" from a Kaiming-uniform draw (seed 42)
+    scaled by sqrt(2).  The head keeps the dtype and device of the projection it replaces.  The reference spells the
+    keyword `init_sceheme` (:96); both spellings are accepted."""
     import math
+
+    if init_scheme is not None and init_sceheme is not None and init_scheme != init_sceheme:
+        raise ValueError("init_scheme and init_sceheme name different schemes")
+    init_scheme = init_scheme if init_scheme is not None else (init_sceheme if init_sceheme is not None else "zeros")
 
     out = transformer.output
     old = out.weight
@@ -452,14 +520,15 @@ def init_random_(model: nn.Module, seed: int = 1234, std: float = 0.02, device=N
 
 
 def random_quantized_transformer(config: ModelArgs, mode: str, groupsize: int = 128, device="cuda", seed: int = 1234,
-                                 std: float = 0.02, reward_head_rows: int = 0) -> nn.Module:
+                                 std: float = 0.02, reward_head_rows: int = 0, seed_on: str = "device") -> nn.Module:
     """Random-init model of the given shape whose linears are already quantized, built layer by layer on
     the GPU: each bf16 weight ~ N(0, std) exists only long enough to be quantized by this package's
     kernels, so a 34B-parameter model never needs its bf16 form in memory.
 
     mode "int4": WeightOnlyInt4Linear (groupsize, inner_k_tiles 8); mode "int8": WeightOnlyInt8Linear;
     mode "bf16": plain nn.Linear.  `reward_head_rows` > 0 wraps the backbone in a RewardModel with that many
-    head rows."""
+    head rows.  seed_on "cpu": the values come from a CPU torch.Generator (the same on every machine, about 8 s per
+    billion parameters); "device": from the GPU's generator (fast; the same for one GPU model and torch build)."""
     import importlib
 
     qz = importlib.import_module(__package__ + ".quantize")  # the package attribute `quantize` is the function
@@ -474,9 +543,12 @@ def random_quantized_transformer(config: ModelArgs, mode: str, groupsize: int = 
         qz.WeightOnlyInt8QuantHandler(model).convert_for_runtime()
     else:
         assert mode == "bf16", mode
-    gen = torch.Generator(device=dev).manual_seed(seed)
+    assert seed_on in ("cpu", "device"), seed_on
+    gen = torch.Generator(device="cpu" if seed_on == "cpu" else dev).manual_seed(seed)
 
     def rand_bf16(shape):
+        if seed_on == "cpu":
+            return torch.randn(shape, generator=gen, dtype=torch.float32).mul_(std).to(torch.bfloat16).to(dev)
         return (torch.randn(shape, generator=gen, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
 
     for _, mod in model.named_modules():

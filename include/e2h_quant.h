@@ -125,7 +125,12 @@ int e2h_int4_dequantize_codes(const int32_t *codes, const uint16_t *scales, cons
  *   workspace  optional scratch of workspace_bytes bytes (16-byte aligned; e2h_workspace_bytes() is the
  *              recommended size) that lets small problems split K across workgroups.  It must be zero
  *              when first used and is left zeroed where it matters by every launch; launches that share
- *              it must be ordered on one stream.  NULL / 0 selects the single-slice kernels. */
+ *              it must be ordered on one stream.  NULL / 0 selects the single-slice kernels.
+ * Every kernel behind this entry point forms exact bf16 x code products and applies scale and zero per group in
+ * float32, so a row's result does not depend on how many rows share the call.  Only with
+ * e2h_set_option("int4_gemm_tile", 256) calls of more than 64 rows (k % 256 == 0, g <= 128, ikt 8) run a kernel that
+ * rounds every weight to bfloat16 first (the arithmetic of the kernel the reference calls; 15-20 % faster at thousands
+ * of rows): results then differ from the default by that rounding, for every row of such a call alike. */
 int e2h_int4_mm(const uint16_t *x, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y,
                 int64_t m, int64_t n, int64_t k, int groupsize, int inner_k_tiles, void *workspace,
                 int64_t workspace_bytes, void *stream);
@@ -219,7 +224,9 @@ int e2h_add_rmsnorm(const uint16_t *x, const uint16_t *delta, const uint16_t *we
  * value e2h_int4_mm stores for the same operands -- before h_out = bf16(x + delta), y = RMSNorm(h_out).
  * e2h_int4_mm_partial_slices returns the number of slices the library uses for a shape (>= 1; it depends on the shape
  * and on e2h_set_option only), or a negative status for shapes this form does not take; e2h_int4_mm_partials rejects
- * any other `slices`.  No workspace is involved.
+ * any other `slices`.  No workspace is involved.  The bit-for-bit statement holds for e2h_int4_mm called with a workspace
+ * of at least e2h_workspace_bytes() and default options; with a smaller or no workspace, or with launch-geometry options
+ * set, e2h_int4_mm may split K differently (or not at all) and the two then agree to float32 rounding only.
  * The int8 pair (WeightOnlyInt8Linear.forward, models/quantize.py:428-429; K % 128 == 0, 16-byte aligned rows) hands on the
  * unscaled sums; col_scales [n] bf16 (NULL for int4) makes the consumer form delta = bf16(bf16(sum) * scale[column]), the
  * linear's two roundings. */
@@ -232,6 +239,84 @@ int e2h_int8_mm_partials(const uint16_t *x, const int8_t *q, float *partials, in
 int e2h_add_rmsnorm_partials(const uint16_t *x, const float *partials, int slices, const uint16_t *col_scales,
                              const uint16_t *weight, uint16_t *h_out, uint16_t *y, int64_t rows, int64_t dim, float eps,
                              void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Decode batches on staged activations.  The single-token steps of the decode loop (reference
+ * inference_generate.py:123-157, decode_one_token :110-120) give every quantized linear at most a few dozen rows;
+ * these entry points are linear_forward_int4 (reference :445-453) and its callers for that case with the activations
+ * handed from kernel to kernel in matrix-core operand order instead of row-major [m, k]:
+ *
+ *   staged buffer for m rows (1 <= m <= 64) of k values (k % 128 == 0), mpad = m rounded up to 16,
+ *   e2h_int4_staged_bytes(m, k) = mpad*k*2 + (k/128)*mpad*32 bytes, 16-byte aligned:
+ *     bf16 [k/32][mpad][32]   the 64-byte piece of row r and 32-wide k segment p; inside it dword 4j + i holds the
+ *                             row's dwords j + 4i of the segment (values k = 32p + 2(j+4i), +1) -- the k order of the
+ *                             packed weight words, so a matrix-core lane loads its operand with one 16-byte load;
+ *     f32  [k/128][mpad][8]   sums over each run of 16 consecutive k (balanced tree in index order).
+ *   Rows m .. mpad-1 may hold anything.
+ *
+ * Common limits: inner_k_tiles == 8 weights, g in {32, 64, 128}, n % 16 == 0, k % 128 == 0, 1 <= m <= 64, and a
+ * launch geometry for the shape (e2h_int4_mm_staged_supported tells; every 7B / 34B linear has one) -- otherwise
+ * E2H_ERR_BAD_SHAPE, and the row-major entry points above take the call.  Results: float32 accumulation of exact
+ * products, scale and zero applied per group in float32, fixed summation order (run-to-run identical); they agree with
+ * the row-major entry points to bfloat16 rounding of the result, not bit for bit (the sums over K are split differently).
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Size of a staged buffer (see above), or a negative status. */
+int64_t e2h_int4_staged_bytes(int64_t m, int64_t k);
+
+/* x [m, k] bf16 row-major -> staged (one pass; padding rows are written as zeros).  No reference counterpart: it is the
+ * layout conversion for activations that do not come from one of the producing kernels below. */
+int e2h_int4_stage_x(const uint16_t *x, void *staged, int64_t m, int64_t k, void *stream);
+
+/* 1 if a staged decode-batch kernel exists for the shape and epilogue (0 = e2h_int4_mm_staged, 1 = _silu_gate,
+ * 2 = _rope_kv, 3 = _partials), else 0. */
+int e2h_int4_mm_staged_supported(int64_t m, int64_t n, int64_t k, int groupsize, int epilogue);
+
+/* linear_forward_int4, reference :445-453: y [m, n] bf16 = staged x times the packed weight. */
+int e2h_int4_mm_staged(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y, int64_t m,
+                       int64_t n, int64_t k, int groupsize, void *stream);
+
+/* The same product left as float32 sums over `slices` contiguous parts of K, partials [slices, m, n], for
+ * e2h_add_rmsnorm_staged to add in slice order (the wo / w2 projections of a decoder block, reference
+ * models/model.py:279-283).  e2h_int4_mm_staged_partial_slices returns the library's slice count for the shape (>= 1) or
+ * a negative status; any other `slices` is rejected. */
+int e2h_int4_mm_staged_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize);
+int e2h_int4_mm_staged_partials(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, float *partials,
+                                int64_t m, int64_t n, int64_t k, int groupsize, int slices, void *stream);
+
+/* F.silu(w1(x)) * w3(x) (FeedForward.forward, reference models/model.py:359-360) with the rounding points of
+ * e2h_int4_mm_silu_gate.  y [m, n] bf16 row-major and / or staged_out, the result in staged form for the w2 projection
+ * (n % 128 == 0 then); at least one of the two must be given. */
+int e2h_int4_mm_staged_silu_gate(const void *staged, const int32_t *packed_gate, const uint16_t *sz_gate, const int32_t *packed_up,
+                                 const uint16_t *sz_up, uint16_t *y, void *staged_out, int64_t m, int64_t n, int64_t k,
+                                 int groupsize, void *stream);
+
+/* e2h_int4_mm_rope_kv on staged activations: fused q|k|v projection, RoPE, cache write (reference models/model.py:321-333
+ * with :400-412 and :121-129); arguments as there. */
+int e2h_int4_mm_staged_rope_kv(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, const uint16_t *freqs_cis,
+                               uint16_t *q_out, uint16_t *k_cache, uint16_t *v_cache, const int64_t *input_pos, int64_t batch,
+                               int64_t n_head, int64_t n_kv_head, int64_t head_dim, int64_t cache_len, int64_t k, int groupsize,
+                               void *stream);
+
+/* RMSNorm (reference models/model.py:363-377) with the optional residual add of TransformerBlock.forward (:279-282) in
+ * front -- e2h_rmsnorm, e2h_add_rmsnorm and e2h_add_rmsnorm_partials in one entry point -- whose normalised rows go to y
+ * (row-major, may be NULL) and / or to `staged` (may be NULL; rows <= 64 and dim % 128 == 0 then).  Exactly as those
+ * three: delta bf16 [rows, dim] or partials float32 [slices, rows, dim] (col_scales as there) or neither; h_out is
+ * required with delta / partials and unused otherwise.  The staged values are bit for bit the values of y. */
+int e2h_add_rmsnorm_staged(const uint16_t *x, const uint16_t *delta, const float *partials, int slices, const uint16_t *col_scales,
+                           const uint16_t *weight, uint16_t *h_out, uint16_t *y, void *staged, int64_t rows, int64_t dim, float eps,
+                           void *stream);
+
+/* e2h_decode_attention whose result [batch, n_head * head_dim] goes to `out` (row-major, may be NULL) and / or to
+ * `staged` (may be NULL), the input of the output projection; batch <= 64 and n_head * head_dim % 128 == 0 with staged. */
+int e2h_decode_attention_staged(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *out, void *staged,
+                                const int64_t *input_pos, const int64_t *left_pad_mask_pos, int64_t batch, int64_t n_head,
+                                int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale, void *stream);
+
+/* Measurement aid, no reference counterpart: one launch of 256 workgroups that only reads `bytes` (a multiple of 16,
+ * < 4 GB) of device memory at src with streaming 16-byte loads and writes nothing (sink may be NULL).  It is the floor
+ * of what a launch that has to read that many bytes of weights can cost on this machine; bytes == 0 is an empty launch. */
+int e2h_stream_read_probe(const void *src, int64_t bytes, uint32_t *sink, void *stream);
 
 /* apply_rotary_emb (reference :400-412) on the q and k parts of a fused qkv row + KVCache.update (:121-129) for
  * one new token per sequence.  qkv [batch, (n_head + 2 n_kv_head) * head_dim]; freqs_cis [positions, head_dim/2, 2]

@@ -272,6 +272,7 @@ def test_decode_step_with_deferred_slices_equals_the_step_without(bsz, mode, mon
     real = getattr(ops, name)
     monkeypatch.setattr(ops, name, lambda *a, **k: (calls.append(a[-1]), real(*a, **k))[1])
     logits = {}
+    monkeypatch.setattr(model_mod, "STAGED_DECODE", False)  # this test is about the row-major kernels' K-slice hand-over
     for defer in (False, True):
         model_mod.DEFER_SPLIT_K = defer
         try:
@@ -296,3 +297,38 @@ def test_decode_step_with_deferred_slices_equals_the_step_without(bsz, mode, mon
         finally:
             model_mod.DEFER_SPLIT_K = True
     assert torch.equal(logits[True], logits[False])
+
+
+def test_staged_decode_step_agrees_with_the_row_major_fused_step(monkeypatch):
+    """The single-token step on staged activations (model.STAGED_DECODE) against the same step on the row-major fused
+    kernels, two layers of the 7B shape at 32 and 5 rows: same arithmetic up to the order of the float32 sums over K, so the
+    logits agree to bfloat16 rounding noise; the staged step replayed from a HIP graph equals its eager run bit for bit."""
+    import easy_to_hard_amd.model as model_mod
+    from easy_to_hard_amd.model import ModelArgs, random_quantized_transformer
+
+    cfg = ModelArgs.from_name("7B")
+    cfg.n_layer = 2
+    model = random_quantized_transformer(cfg, "int4", 128, device=DEV, seed=7)
+    t = 7
+    for bsz in (32, 5):
+        prompt = torch.randint(0, cfg.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(4)).to(DEV)
+        logits = {}
+        for staged in (False, True):
+            monkeypatch.setattr(model_mod, "STAGED_DECODE", staged)
+            model.max_seq_length = -1
+            model.setup_caches(bsz, 32)
+            assert model.staged_step_supported(bsz) == staged
+            cur = prefill(model, prompt, torch.arange(0, t, device=DEV))
+            out = []
+            for i in range(3):
+                lg = model(cur, torch.tensor([t + i], device=DEV))
+                out.append(lg[:, -1].clone())
+                cur = torch.argmax(lg[:, -1].float(), dim=-1, keepdim=True)
+            logits[staged] = torch.stack(out).float()
+        err = (logits[True] - logits[False]).abs().max() / logits[False].abs().max()
+        assert err <= 2e-2, err
+        stepper = GraphedDecodeStep(model, bsz, DEV)
+        prefill(model, prompt, torch.arange(0, t, device=DEV))
+        first = torch.argmax(logits[True][0], dim=-1, keepdim=True)
+        tok = stepper.step(first, torch.tensor([t + 1], device=DEV)).clone()
+        assert torch.equal(tok, torch.argmax(logits[True][1], dim=-1, keepdim=True))
