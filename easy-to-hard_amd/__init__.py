@@ -5,6 +5,9 @@ libe2h_quant.so (C ABI: include/e2h_quant.h) and are loaded on first use.
 """
 
 from . import _lib, ops  # noqa: F401
+from . import _traced as _traced
+
+_traced.install()  # e2h:: custom ops behind the public names of ops.py while a torch.compile trace is taken
 from .quantize import (  # noqa: F401
     QuantHandler,
     WeightOnlyInt4Linear,

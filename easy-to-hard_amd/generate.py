@@ -19,7 +19,7 @@ from . import ops
 def greedy_token(logits: Tensor) -> Tensor:
     """argmax over the vocabulary of the last position, in float32 -> [B, 1] int64."""
     last = logits[:, -1]
-    if last.is_cuda and last.dtype == torch.bfloat16 and not torch.compiler.is_compiling():
+    if last.is_cuda and last.dtype == torch.bfloat16:
         return ops.argmax_rows(last)
     return torch.argmax(last.float(), dim=-1, keepdim=True)
 

@@ -33,7 +33,7 @@ STAGED_MAX_ROWS = 32         # beyond one 32-row slab the row-major kernels are 
 
 
 def _fusable(t: Tensor) -> bool:
-    return FUSED_DECODE and t.is_cuda and t.dtype == torch.bfloat16 and not torch.compiler.is_compiling()
+    return FUSED_DECODE and t.is_cuda and t.dtype == torch.bfloat16
 
 
 @dataclass
@@ -256,7 +256,7 @@ class FeedForward(nn.Module):
         w1, w3 = self.w1, self.w3
         if not (FUSED_DECODE and FUSE_GATE and isinstance(w1, WeightOnlyInt4Linear) and isinstance(w3, WeightOnlyInt4Linear)):
             return False
-        if w1.padding or w3.padding or torch.compiler.is_compiling():
+        if w1.padding or w3.padding:
             return False
         return ops.int4_gate_supported(x, w1, w3)
 
@@ -264,7 +264,7 @@ class FeedForward(nn.Module):
         w1, w3 = self.w1, self.w3
         if not (FUSED_DECODE and FUSE_GATE and isinstance(w1, WeightOnlyInt8Linear) and isinstance(w3, WeightOnlyInt8Linear)):
             return False
-        return not torch.compiler.is_compiling() and ops.int8_gate_supported(x, w1, w3)
+        return ops.int8_gate_supported(x, w1, w3)
 
     def forward(self, x: Tensor, defer_output: bool = False) -> Tensor:
         if defer_output and self._gate_fusable_int8(x):
@@ -393,7 +393,7 @@ class Transformer(nn.Module):
     def staged_step_supported(self, rows: int) -> bool:
         """True when a single-token step of `rows` sequences runs on the decode-batch int4 kernels with staged activations
         (an int4 model on the GPU with bfloat16 norms and caches set up, at most STAGED_MAX_ROWS sequences)."""
-        if not (FUSED_DECODE and STAGED_DECODE and FUSE_GATE and FUSE_ROPE_PROJECTION and DEFER_SPLIT_K) or torch.compiler.is_compiling():
+        if not (FUSED_DECODE and STAGED_DECODE and FUSE_GATE and FUSE_ROPE_PROJECTION and DEFER_SPLIT_K):
             return False
         if not (1 <= rows <= STAGED_MAX_ROWS and self.config.dim % 128 == 0 and self.kv_cache_enabled and self.freqs_cis is not None):
             return False

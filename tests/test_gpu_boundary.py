@@ -41,24 +41,53 @@ def test_quantized_modules_trace_under_fullgraph_compile_and_match_eager():
             assert torch.equal(compiled(x[:1, :1]), lin(x[:1, :1]))   # another shape retraces
 
 
-def test_decode_step_traces_under_fullgraph_compile():
-    """One decode step of a quantized model under torch.compile(fullgraph=True): the trace takes the stock-op branches
-    around the linears and the custom ops for the linears; logits agree with the eager fused step to bfloat16 noise and the
-    greedy token is the same."""
-    model = _tiny_int4()
-    bsz, t = 3, 9
+def _compiled_step_equals_graphed_step(model, bsz, t):
+    """The reference decodes through torch.compile(mode="reduce-overhead", fullgraph=True) (inference_generate.py:346-349).
+    Here: the model under torch.compile(backend="aot_eager", fullgraph=True) -- a trace with fake tensors through the
+    registered e2h:: ops, any graph break is an error -- must run the very kernels of the HIP-graph replayed step: same
+    logits as the eager step and the same next token as GraphedDecodeStep, bit for bit."""
     model.setup_caches(bsz, 32)
     prompt = torch.randint(0, model.config.vocab_size, (bsz, t), generator=torch.Generator().manual_seed(5)).to(DEV)
     pos = torch.arange(0, t, device=DEV)
+    step_pos = torch.tensor([t], device=DEV)
     with torch.no_grad():
         cur = prefill(model, prompt, pos)
-        step_pos = torch.tensor([t], device=DEV)
         eager = model(cur, step_pos).clone()
         prefill(model, prompt, pos)
         compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
-        traced = compiled(cur, step_pos)
-    err = (traced.float() - eager.float()).abs().max() / eager.float().abs().max()
-    assert err <= 2e-2, float(err)
+        traced = compiled(cur, step_pos).clone()
+        assert torch.equal(traced, eager)
+        stepper = GraphedDecodeStep(model, bsz, DEV)
+        prefill(model, prompt, pos)
+        replay = stepper.step(cur, step_pos).clone()
+        assert torch.equal(replay, torch.argmax(traced[:, -1].float(), dim=-1, keepdim=True))
+        # a second traced step (the first one's token, next position) against the eager one, caches included
+        nxt_pos = torch.tensor([t + 1], device=DEV)
+        prefill(model, prompt, pos)
+        model(cur, step_pos)
+        want = model(replay, nxt_pos).clone()
+        prefill(model, prompt, pos)
+        compiled(cur, step_pos)
+        assert torch.equal(compiled(replay, nxt_pos), want)
+
+
+@pytest.mark.parametrize("name", ["tiny-test", "tiny-gqa-test"])
+def test_fused_decode_step_under_fullgraph_compile_equals_the_graphed_step(name):
+    _compiled_step_equals_graphed_step(_tiny_int4(name), 3, 9)
+
+
+@pytest.mark.parametrize("mode", ["int4", "int8"])
+def test_7b_shaped_decode_step_under_fullgraph_compile_equals_the_graphed_step(mode):
+    """Two layers of the 7B shape at 32 rows: the int4 model takes the staged decode-batch kernels (asserted), the int8
+    model the row-major fused kernels, traced exactly as they run eagerly."""
+    from easy_to_hard_amd.model import ModelArgs, random_quantized_transformer
+
+    cfg = ModelArgs.from_name("7B")
+    cfg.n_layer = 2
+    model = random_quantized_transformer(cfg, mode, 128, device=DEV, seed=7)
+    model.setup_caches(32, 32)
+    assert model.staged_step_supported(32) == (mode == "int4")
+    _compiled_step_equals_graphed_step(model, 32, 7)
 
 
 @pytest.mark.parametrize("name", ["tiny-test", "tiny-gqa-test"])
