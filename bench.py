@@ -31,9 +31,10 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per dequant-GEMV launch (fetched + written) from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --gemv-only`, scaled by a 256 MiB copy; the summary with the commands is in
-# profiles/int4_skinny_mm_7b_decode_bs32.md.  Counters cannot be read from inside this process, so the figure is
-# recorded here for the configuration it was measured on and reported as null for any other.
-MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32, "int4_skinny_mm_kernel"): 33_440_000}
+# profiles/int4_staged_mm_7b_decode_bs32.md (int4_skinny_mm_7b_decode_bs32.md for the row-major kernels).  Counters cannot be read from inside this process, so the figure is
+# recorded here for the configuration and kernel set it was measured on and reported as null for any other.
+MEASURED_TRAFFIC_BYTES = {("7B", "int4", 128, 32, "int4_skinny_mm_kernel"): 33_440_000,
+                          ("7B", "int4", 128, 32, "int4_staged_mm_kernel"): 32_370_000}
 
 
 def parse_args():

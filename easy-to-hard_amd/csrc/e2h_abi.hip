@@ -108,6 +108,11 @@ extern "C" int e2h_set_option(const char *name, int value) {
     o.int8_gemm_tile = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "staged_tiles") || !strcmp(name, "staged_slices")) {
+    if (value < 0 || value > 16) return E2H_ERR_BAD_OPTION;
+    (name[7] == 't' ? o.staged_tiles : o.staged_slices) = value;
+    return E2H_OK;
+  }
   if (!strcmp(name, "attention_no_mfma")) {
     o.attention_no_mfma = value != 0;
     return E2H_OK;

@@ -401,7 +401,7 @@ struct Geometry {
 struct Inst {
   int t, c, dw, dx;
 };
-constexpr Inst kPlainInsts[] = {{3, 4, 2, 2}, {4, 4, 2, 2}, {8, 4, 1, 1}, {6, 4, 2, 1}, {2, 2, 2, 2}, {4, 2, 2, 2}, {4, 1, 1, 1}, {4, 3, 3, 1}, {4, 8, 2, 1}, {8, 8, 1, 1}};
+constexpr Inst kPlainInsts[] = {{3, 4, 2, 2}, {4, 4, 2, 2}, {8, 4, 1, 1}, {6, 4, 2, 1}, {2, 2, 2, 2}, {4, 2, 2, 2}, {6, 2, 2, 2}, {4, 1, 1, 1}, {4, 3, 3, 1}, {4, 8, 2, 1}, {8, 8, 1, 1}, {2, 1, 1, 1}};
 constexpr Inst kGateInsts[] = {{6, 4, 2, 1}, {4, 4, 2, 2}, {8, 4, 1, 1}, {6, 8, 1, 1}, {8, 8, 1, 1}};
 
 // instantiations that do not fit the 256 vector registers of a wave (they would run, slowly, out of scratch memory):
@@ -415,12 +415,15 @@ inline bool fits_registers(int groupsize, const Inst &in) {
 template <int NI>
 bool pick(const Inst (&insts)[NI], bool gate, int groupsize, int tiles16, int kt, int slabs, int max_slices, Geometry *best) {
   long best_cost = -1;
+  const int want_t = options().staged_tiles, want_s = options().staged_slices;  // experiments: force a geometry
   for (int s = 1; s <= max_slices; s *= 2) {
+    if (want_s && s != want_s) continue;
     if (s > kt) break;
     const int per_slice = (kt + s - 1) / s;  // the longest slice
     const int c_need = (per_slice + kWaves - 1) / kWaves;
     for (const Inst &in : insts) {
       if (in.c != c_need || !fits_registers(groupsize, in)) continue;
+      if (want_t && !gate && in.t != want_t) continue;
       const int tc = gate ? in.t / 2 : in.t;
       const long wgs = static_cast<long>((tiles16 + tc - 1) / tc) * s * slabs;
       const long rounds = (wgs + kCUs - 1) / kCUs;
@@ -451,7 +454,7 @@ int dispatch_inst(const StagedArgs &a, const Geometry &g, hipStream_t stream) {
     E2H_ST_CASE(6, 4, 2, 1) E2H_ST_CASE(4, 4, 2, 2) E2H_ST_CASE(8, 4, 1, 1) E2H_ST_CASE(6, 8, 1, 1) E2H_ST_CASE(8, 8, 1, 1)
   } else {
     E2H_ST_CASE(3, 4, 2, 2) E2H_ST_CASE(4, 4, 2, 2) E2H_ST_CASE(8, 4, 1, 1) E2H_ST_CASE(6, 4, 2, 1) E2H_ST_CASE(2, 2, 2, 2)
-    E2H_ST_CASE(4, 2, 2, 2) E2H_ST_CASE(4, 1, 1, 1) E2H_ST_CASE(4, 3, 3, 1) E2H_ST_CASE(4, 8, 2, 1) E2H_ST_CASE(8, 8, 1, 1)
+    E2H_ST_CASE(4, 2, 2, 2) E2H_ST_CASE(6, 2, 2, 2) E2H_ST_CASE(4, 1, 1, 1) E2H_ST_CASE(2, 1, 1, 1) E2H_ST_CASE(4, 3, 3, 1) E2H_ST_CASE(4, 8, 2, 1) E2H_ST_CASE(8, 8, 1, 1)
   }
 #undef E2H_ST_CASE
   return E2H_ERR_BAD_SHAPE;

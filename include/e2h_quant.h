@@ -42,7 +42,7 @@ const char *e2h_status_string(int status);
 /* Tuning knobs for experiments: launch-geometry overrides such as "int4_rows_per_wave", "int4_k_slices", "int4_k_groups",
  * "int4_col_waves", "int8_rows_per_wave", "int8_k_groups", "int8_k_slices", "int8_force_generic", "row_tiles", "int4_no_xsum",
  * "int4_no_gemm32", "int4_gemm32_min_rows", "int4_gemm_tile", "int8_gemm_tile", "int8_gemm_waves", "int8_gemm_wave_cols", "attention_waves",
- * "attention_no_mfma";
+ * "attention_no_mfma", "staged_tiles", "staged_slices";
  * value 0 restores the built-in heuristic.  Not thread safe; set before launching. */
 int e2h_set_option(const char *name, int value);
 
