@@ -231,24 +231,29 @@ def measure_launch_floor(model, batch, reps):
 
     dev = torch.device("cuda", 0)
     lib = _lib.load()
-    sizes = []  # weight + qparam bytes of every launch of a step (w1 and w3 share a launch)
+    sizes = []  # (name, weight + qparam bytes, activation bytes) of every launch of a step (w1 and w3 share a launch)
     for blk in model.layers:
         att, ff = blk.attention, blk.feed_forward
         wb = lambda m: algorithmic_bytes(m, 0)
-        sizes += [("wqkv", wb(att.wqkv)), ("wo", wb(att.wo)), ("w1+w3", wb(ff.w1) + wb(ff.w3)), ("w2", wb(ff.w2))]
-    sizes.append(("output", algorithmic_bytes(model.output, 0)))
+        xb = lambda m: batch * m.in_features * 2
+        sizes += [("wqkv", wb(att.wqkv), xb(att.wqkv)), ("wo", wb(att.wo), xb(att.wo)), ("w1+w3", wb(ff.w1) + wb(ff.w3), xb(ff.w1)),
+                  ("w2", wb(ff.w2), xb(ff.w2))]
+    sizes.append(("output", algorithmic_bytes(model.output, 0), batch * model.output.in_features * 2))
     region = torch.empty(3 << 30, dtype=torch.uint8, device=dev).fill_(3)
+    shared = torch.empty(max(x for _, _, x in sizes) + 16, dtype=torch.uint8, device=dev).fill_(5)
     stream = lambda: ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
     def timed(launches):
-        """launches: list of byte counts; returns the average microseconds per launch"""
+        """launches: list of (weight bytes, shared activation bytes); returns the average microseconds per launch"""
         def one_pass():
             off = 0
-            for nbytes in launches:
+            for nbytes, xbytes in launches:
                 nbytes -= nbytes % 16
+                xbytes -= xbytes % 16
                 if off + nbytes > region.numel():
                     off = 0
-                rc = lib.e2h_stream_read_probe(ctypes.c_void_p(region.data_ptr() + off), nbytes, None, stream())
+                rc = lib.e2h_stream_read_probe(ctypes.c_void_p(region.data_ptr() + off), nbytes, ctypes.c_void_p(shared.data_ptr()), xbytes,
+                                               None, stream())
                 assert rc == 0, rc
                 off += (nbytes + 4095) // 4096 * 4096
         side = torch.cuda.Stream(device=dev)
@@ -270,16 +275,22 @@ def measure_launch_floor(model, batch, reps):
         return start.elapsed_time(stop) * 1e3 / (reps * len(launches))
 
     per_size = {}
-    for name, nbytes in sizes:
+    for name, nbytes, xbytes in sizes:
         if name not in per_size:
-            per_size[name] = {"bytes": nbytes, "us": round(timed([nbytes] * 64), 2)}
-    empty_us = round(timed([0] * 256), 2)
-    step_us = timed([b for _, b in sizes]) * len(sizes)
-    total_bytes = sum(b for _, b in sizes)
+            per_size[name] = {"bytes": nbytes, "us": round(timed([(nbytes, 0)] * 64), 2), "activation_bytes": xbytes,
+                              "us_with_activations_read_by_every_workgroup": round(timed([(nbytes, xbytes)] * 64), 2)}
+    empty_us = round(timed([(0, 0)] * 256), 2)
+    step_us = timed([(b, 0) for _, b, _ in sizes]) * len(sizes)
+    step_x_us = timed([(b, x) for _, b, x in sizes]) * len(sizes)
+    total_bytes = sum(b for _, b, _ in sizes)
     return {"empty_launch_us": empty_us, "per_launch": per_size, "launches_per_step": len(sizes),
             "read_only_ms_per_step": round(step_us * 1e-3, 4), "weight_bytes_per_step": total_bytes,
             "hbm_frac_of_a_read_only_step": round(total_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "note": "a launch-per-linear decode step cannot spend less time in its quantized linears than read_only_ms_per_step"}
+            "read_only_ms_per_step_with_activations": round(step_x_us * 1e-3, 4),
+            "hbm_frac_of_a_read_only_step_with_activations": round(total_bytes / (step_x_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "note": "a launch-per-linear decode step cannot spend less time in its quantized linears than read_only_ms_per_step; "
+                    "with_activations: every workgroup of the read-only launch also reads the batch's activations (from L2), as every CU of "
+                    "a decode-batch matmul must"}
 
 
 def stock_int4_operands(mod):

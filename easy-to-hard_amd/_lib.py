@@ -55,7 +55,7 @@ _SIGNATURES = {
     "e2h_int4_mm_staged_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),
     "e2h_int4_mm_staged_rope_kv": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, _P]),
     "e2h_add_rmsnorm_staged": (c_int, [_P, _P, _P, c_int, _P, _P, _P, _P, _P, c_int64, c_int64, c_float, _P]),
-    "e2h_stream_read_probe": (c_int, [_P, c_int64, _P, _P]),
+    "e2h_stream_read_probe": (c_int, [_P, c_int64, _P, c_int64, _P, _P]),
     "e2h_decode_attention_staged": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, _P]),
 }
 

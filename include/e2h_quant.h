@@ -314,9 +314,11 @@ int e2h_decode_attention_staged(const uint16_t *q, const uint16_t *k_cache, cons
                                 int64_t n_kv_head, int64_t cache_len, int64_t head_dim, float scale, void *stream);
 
 /* Measurement aid, no reference counterpart: one launch of 256 workgroups that only reads `bytes` (a multiple of 16,
- * < 4 GB) of device memory at src with streaming 16-byte loads and writes nothing (sink may be NULL).  It is the floor
- * of what a launch that has to read that many bytes of weights can cost on this machine; bytes == 0 is an empty launch. */
-int e2h_stream_read_probe(const void *src, int64_t bytes, uint32_t *sink, void *stream);
+ * < 2 GB) of device memory at src with streaming 16-byte loads and writes nothing (sink may be NULL).  It is the floor
+ * of what a launch that has to read that many bytes of weights can cost on this machine; bytes == 0 is an empty launch.
+ * With shared_bytes > 0 every workgroup additionally reads all of `shared` (a multiple of 16, < 2 GB): the pattern of
+ * a decode batch's activations, which every CU needs whole next to its share of the weights. */
+int e2h_stream_read_probe(const void *src, int64_t bytes, const void *shared, int64_t shared_bytes, uint32_t *sink, void *stream);
 
 /* apply_rotary_emb (reference :400-412) on the q and k parts of a fused qkv row + KVCache.update (:121-129) for
  * one new token per sequence.  qkv [batch, (n_head + 2 n_kv_head) * head_dim]; freqs_cis [positions, head_dim/2, 2]
