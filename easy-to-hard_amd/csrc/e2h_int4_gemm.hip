@@ -236,23 +236,10 @@ __global__ __launch_bounds__(64 * WR * WC) void int4_gemm32_kernel(const uint16_
   }
 
   // ---- store: lane (h, n) holds column col0 + 32 ct + n, rows 8 (e / 4) + 4 h + e % 4 of each tile -----------
-  if ((reinterpret_cast<uintptr_t>(y) & 15) == 0) {  // N % 8 == 0 always holds for the packed layout
-    // (the barrier that ended the last chunk left every wave done with the stages)
-    const float no_scale[kCT] = {};
-    store_tiles_via_lds<kRT, kCT, false>(acc, no_scale, lds + wave * TileStore<kCT>::kBytesPerWave, y, row0, col0, M, N, lane);
-    return;
-  }
-#pragma unroll
-  for (int ct = 0; ct < kCT; ++ct) {
-    const int col = col0 + 32 * ct + n;
-#pragma unroll
-    for (int rt = 0; rt < kRT; ++rt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = row0 + 32 * rt + 8 * (e >> 2) + 4 * h + (e & 3);
-        if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = f32_to_bf16_rne(acc[ct][rt][e]);
-      }
-  }
+  // (the barrier that ended the last chunk left every wave done with the stages)
+  const float no_scale[kCT] = {};
+  store_tiles_via_lds<kRT, kCT, false>(acc, no_scale, lds + wave * TileStore<kCT>::kBytesPerWave, y, row0, col0, M, N, lane,
+                                    (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0);
 }
 
 }  // namespace

@@ -33,7 +33,11 @@ namespace {
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kFragA = 1024 + 32;  // one 32-row x 16-k A fragment block in LDS (64 lanes x 16 B) + skew
+// One 32-row x 16-k A fragment block in LDS: lane (h, r) at h * kHalfA + 16 r.  A 16-lane group of the staging stores
+// covers 2 rows x 8 pieces = 4 steps x 2 halves, 32 bytes each; with these strides (5 * 32 and 128 mod 256) the 16 stores
+// fall into 16 different 16-byte bank groups of the 256-byte LDS row, as the fragment reads (256 contiguous bytes per
+// 16 lanes) always do.
+constexpr int kFragA = 1184, kHalfA = 640;
 
 template <int G>
 __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp,
@@ -85,7 +89,7 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
     row = row < M ? row : M - 1;
     xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + xw * 8) * 2);
   }
-  const int xdst0 = (xw >> 1) * kFragA + ((xw & 1) * 32 + xr0) * 16;  // pass i covers row tile i
+  const int xdst0 = (xw >> 1) * kFragA + (xw & 1) * kHalfA + xr0 * 16;  // pass i covers row tile i
 
   // ---- weights: byte offset of piece j = 0 of this lane's column inside block 0; (scale, zero) column offset
   uint32_t wlane[CT], szlane[CT];
@@ -122,7 +126,7 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
   };
   bf16x8_t af[RT];  // fragment rt is re-read for the next step right after its last MFMA of this one
   auto read_a = [&](int parity, int s, int rt) {
-    return *reinterpret_cast<const bf16x8_t *>(lds + (parity & 1) * kStageX + lane * 16 + (rt * SPC + s) * kFragA);
+    return *reinterpret_cast<const bf16x8_t *>(lds + (parity & 1) * kStageX + h * kHalfA + n * 16 + (rt * SPC + s) * kFragA);
   };
 
   // ---- conversion of one operand in four parts (dword j each): unpack, two float32 FMAs, one packed round ----------
@@ -212,23 +216,10 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
   }
 
   // ---- store: lane (h, n) holds column col0 + 32 ct + n, rows 8 (e / 4) + 4 h + e % 4 of each tile -----------------
-  if ((reinterpret_cast<uintptr_t>(y) & 15) == 0) {  // N % 8 == 0 always holds for the packed layout
-    lds_barrier();  // the staging stages are dead from here on
-    const float no_scale[CT] = {};
-    store_tiles_via_lds<RT, CT, false>(acc, no_scale, lds + wave * TileStore<CT>::kBytesPerWave, y, row0, col0, M, N, lane);
-    return;
-  }
-#pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    const int col = col0 + 32 * ct + n;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = row0 + 32 * rt + 8 * (e >> 2) + 4 * h + (e & 3);
-        if (row < M && col < N) y[static_cast<size_t>(row) * N + col] = f32_to_bf16_rne(acc[ct][rt][e]);
-      }
-  }
+  lds_barrier();  // the staging stages are dead from here on
+  const float no_scale[CT] = {};
+  store_tiles_via_lds<RT, CT, false>(acc, no_scale, lds + wave * TileStore<CT>::kBytesPerWave, y, row0, col0, M, N, lane,
+                                    (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0);
 }
 
 }  // namespace

@@ -33,7 +33,8 @@ __device__ __forceinline__ bf16x8_t unpack_word(uint32_t w, const UnpackConsts &
 // 32-row slab goes through a wave-private LDS tile (32 rows x 32 CT columns, row stride kTileStride bytes) and leaves
 // as 16-byte pieces of output rows.  Rounding uses the packed hardware convert (round to nearest even, two values per
 // instruction).  kScale: the int8 contract y = bf16(bf16(acc) * scale[column]); otherwise y = bf16(acc).
-// Needs N % 8 == 0 and a 16-byte aligned y (the caller checks and otherwise stores element-wise).
+// pieces (uniform): N % 8 == 0 and y 16-byte aligned, so that every piece is one aligned 16-byte store; otherwise the
+// eight values of a piece leave one by one, bounds-checked against N.
 typedef float e2h_float2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 e2h_bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float e2h_f32x16_t __attribute__((ext_vector_type(16)));
@@ -50,7 +51,8 @@ __device__ __forceinline__ uint32_t pack_bf16x2_rne(float a, float b) {
 
 template <int RT, int CT, bool kScale>
 __device__ __forceinline__ void store_tiles_via_lds(const e2h_f32x16_t (&acc)[CT][RT], const float (&scale)[CT], uint8_t *tile,
-                                                    uint16_t *__restrict__ y, int row0, int col0, int M, int N, int lane) {
+                                                    uint16_t *__restrict__ y, int row0, int col0, int M, int N, int lane,
+                                                    bool pieces) {
   constexpr int kTileStride = TileStore<CT>::kTileStride;
   constexpr int kPiecesPerRow = 4 * CT;             // 16-byte pieces per tile row
   constexpr int kRowsPerPass = 64 / kPiecesPerRow;  // tile rows one 64-lane read covers
@@ -80,7 +82,16 @@ __device__ __forceinline__ void store_tiles_via_lds(const e2h_f32x16_t (&acc)[CT
       const int trow = pass * kRowsPerPass + lane / kPiecesPerRow, piece = lane % kPiecesPerRow;
       const u32x4_t v = *reinterpret_cast<const u32x4_t *>(tile + trow * kTileStride + piece * 16);
       const int row = row0 + 32 * rt + trow, col = col0 + 8 * piece;
-      if (row < M && col < N) *reinterpret_cast<u32x4_t *>(y + static_cast<size_t>(row) * N + col) = v;
+      if (row < M && col < N) {
+        uint16_t *dst = y + static_cast<size_t>(row) * N + col;
+        if (pieces) {
+          *reinterpret_cast<u32x4_t *>(dst) = v;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (col + j < N) dst[j] = static_cast<uint16_t>(v[j >> 1] >> (16 * (j & 1)));
+        }
+      }
     }
   }
 }

@@ -400,7 +400,7 @@ def test_int4_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, g):
     assert (yi.float() - yi2.float()).abs().max().item() <= 2.0 ** -7 * yi2.float().abs().max().item()
 
 
-@pytest.mark.parametrize("tile,waves,wave_cols", [(128, 0, 0), (256, 8, 0), (256, 4, 2), (256, 4, 4)])
+@pytest.mark.parametrize("tile,waves,wave_cols", [(128, 0, 0), (256, 0, 0), (256, 8, 0), (256, 4, 2), (256, 4, 4)])
 @pytest.mark.parametrize("m,n,k", [(65, 1, 128), (130, 272, 1024), (257, 136, 384), (512, 4096, 4096), (300, 2, 4096), (700, 520, 640)])
 def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile, waves, wave_cols):
     """The 32x32-tile int8 kernels (many rows; 128 x 256 and 256 x 256 outputs per workgroup, the latter with eight or four waves) against the oracle, the
