@@ -13,8 +13,12 @@
 //
 // Main loop, v_mfma_f32_32x32x16_bf16 (A = activations, 32 rows; B = weights, 32 columns; 16 k per instruction), k in
 // natural order: lane L = 32 h + n supplies column n0 + n and the eight k values 16 s + 8 h .. + 7 of step s.
-//   Activations are staged per 64-wide k chunk into LDS in fragment order by plain 16-byte copies (double buffered,
-//   one LDS barrier per chunk): the fragment of lane (h, m) for step s is x[m][16 s + 8 h .. + 7].
+//   Activations reach LDS per 64-wide k chunk by 16-byte buffer loads that write LDS directly (lane L of an
+//   instruction lands at base + 16 L; no staging registers, no staging stores), three 32 KB stages: the chunk in use and
+//   two in flight, one barrier per chunk.  1 KB block b holds rows 8 b .. 8 b + 7, 128 bytes each (eight lanes read one
+//   whole row segment); within a row the 16-byte pieces sit at position piece ^ ((row >> 1) & 7), so the fragment read
+//   of 16 consecutive rows at one piece index touches 16 different bank groups.  The fragment of lane (h, m) for step
+//   s is x[m][16 s + 8 h .. + 7] = piece 2 s + h.
 //   Weights never touch LDS.  A packed word (column, j, span p) holds the codes at k = 32 p + 8 i + 2 j + {0, 1} in
 //   nibbles i and i + 4 (i = 0 .. 3), and the checkpoint stores the four spans of a 128-wide k block next to each
 //   other: the lane loads, per column tile and block, the four 16-byte pieces j = 0 .. 3 of its column (32 registers
@@ -33,12 +37,6 @@ namespace {
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-// One 32-row x 16-k A fragment block in LDS: lane (h, r) at h * kHalfA + 16 r.  A 16-lane group of the staging stores
-// covers 2 rows x 8 pieces = 4 steps x 2 halves, 32 bytes each; with these strides (5 * 32 and 128 mod 256) the 16 stores
-// fall into 16 different 16-byte bank groups of the 256-byte LDS row, as the fragment reads (256 contiguous bytes per
-// 16 lanes) always do.
-constexpr int kFragA = 1184, kHalfA = 640;
-
 template <int G>
 __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ wp,
                                                            const uint32_t *__restrict__ sz, uint16_t *__restrict__ y, int M, int N, int K,
@@ -47,11 +45,12 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
   constexpr int CK = 64;               // k per staged activation chunk
   constexpr int SPC = CK / 16;         // MFMA steps per chunk
   constexpr int NGRP = 128 / G;        // quantization groups per 128-wide weight block
-  constexpr int kStageX = RT * SPC * kFragA;
+  constexpr int kStageX = 256 * 128;   // 256 rows x 64 k of bfloat16
   constexpr int kXPieces = 8;          // 256 rows x 8 pieces of 16 bytes per chunk, 256 threads
   static_assert(G == 32 || G == 64 || G == 128, "group sizes of the packed format up to one weight block");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageX];
-  static_assert(2 * kStageX >= 4 * TileStore<CT>::kBytesPerWave, "the output tiles reuse the stages");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[3 * kStageX];
+  static_assert(kStageX >= 4 * TileStore<CT>::kBytesPerWave, "the output tiles reuse a stage");
+  typedef __attribute__((address_space(3))) void lds_void;
 
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
@@ -80,16 +79,18 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[ct][rt][e] = 0.f;
 
-  // ---- activation staging: piece (row, w), k = 8 w .. 8 w + 7, goes to fragment (row tile, step w / 2), lane (w % 2, row % 32)
-  const int xr0 = tid >> 3, xw = tid & 7;
+  // ---- what this lane loads: activation block w + 4 i, row 8 (w + 4 i) + lane / 8, the piece that belongs at position
+  // lane % 8 (the swizzle term ((row >> 1) & 7) is the same for every i)
   uint32_t xsrc[kXPieces];
+  {
+    const int xpiece = (lane & 7) ^ (((lane >> 4) + 4 * wave) & 7);
 #pragma unroll
-  for (int i = 0; i < kXPieces; ++i) {
-    int row = row0 + xr0 + 32 * i;
-    row = row < M ? row : M - 1;
-    xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + xw * 8) * 2);
+    for (int i = 0; i < kXPieces; ++i) {
+      int row = row0 + 8 * (wave + 4 * i) + (lane >> 3);
+      row = row < M ? row : M - 1;
+      xsrc[i] = static_cast<uint32_t>((static_cast<size_t>(row) * K + xpiece * 8) * 2);
+    }
   }
-  const int xdst0 = (xw >> 1) * kFragA + (xw & 1) * kHalfA + xr0 * 16;  // pass i covers row tile i
 
   // ---- weights: byte offset of piece j = 0 of this lane's column inside block 0; (scale, zero) column offset
   uint32_t wlane[CT], szlane[CT];
@@ -114,19 +115,17 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
     w.sz[i / NGRP][i % NGRP] = __builtin_amdgcn_raw_buffer_load_b32(sz_rsrc, szlane[i / NGRP], static_cast<uint32_t>(bb * NGRP + i % NGRP) * N * 4u, 0);
   };
 
-  struct Staged {
-    u32x4_t p[kXPieces];
-  };
-  auto load_piece = [&](Staged &r, int ci, int i) {
+  auto load_piece = [&](int ci, uint32_t stage_off, int i) {  // stage_off: byte offset of the stage that receives chunk ci (uniform)
     const int cc = ci < nchunks ? ci : nchunks - 1;
-    r.p[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, xsrc[i], static_cast<uint32_t>(cc) * (CK * 2), 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (lds_void *)(lds + stage_off + (wave + 4 * i) * 1024), 16, xsrc[i],
+                                             static_cast<uint32_t>(cc) * (CK * 2), 0, 0);
   };
-  auto store_piece = [&](const Staged &r, int parity, int i) {
-    *reinterpret_cast<u32x4_t *>(lds + (parity & 1) * kStageX + xdst0 + i * (SPC * kFragA)) = r.p[i];
-  };
+  uint32_t a_lane[SPC];  // lane (h, r), step s: row r, piece 2 s + h at position (2 s + h) ^ ((r >> 1) & 7)
+#pragma unroll
+  for (int s2 = 0; s2 < SPC; ++s2) a_lane[s2] = static_cast<uint32_t>(n * 128 + (((2 * s2 + h) ^ ((n >> 1) & 7)) << 4));
   bf16x8_t af[RT];  // fragment rt is re-read for the next step right after its last MFMA of this one
-  auto read_a = [&](int parity, int s, int rt) {
-    return *reinterpret_cast<const bf16x8_t *>(lds + (parity & 1) * kStageX + h * kHalfA + n * 16 + (rt * SPC + s) * kFragA);
+  auto read_a = [&](uint32_t stage_off, int s2, int rt) {
+    return *reinterpret_cast<const bf16x8_t *>(lds + stage_off + a_lane[s2] + rt * 4096);
   };
 
   // ---- conversion of one operand in four parts (dword j each): unpack, two float32 FMAs, one packed round ----------
@@ -148,26 +147,31 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
   };
   bf16x8_t wf;  // converted operand of the column tile whose MFMAs come next
 
-  // Slot j = 0 .. 15 of step s of chunk ci (half hf of its weight block), whose register set r holds chunk ci + 1:
+  // Slot j = 0 .. 15 of step s of chunk ci (half hf of its weight block; stage scur, the next chunk in stage snxt, chunk
+  // ci + 2 goes to stage sfar, which every wave left before the previous barrier):
   //   j >= 8 (second column tile, the fragment's last use in this step): activation fragment j - 8 of the next step
-  //   s < 2, j = 0 .. 3: staging store of piece 4 s + j;  j = 4 .. 7: load of that piece of chunk ci + 3
+  //   s < 2, j = 4 .. 7: load 4 s + j - 4 of chunk ci + 2
   //   s = 2 of a block's first half: the eight weight loads (j < 8) and the (scale, zero) loads (j >= 8) of the next block
   // The last step's fragment reads address the next chunk's stage, behind the chunk's only barrier.
-  auto slot_op = [&](int ci, Staged &r, WSet &nxt, int hf, int s, int j) {
+  auto slot_op = [&](int ci, uint32_t scur, uint32_t snxt, uint32_t sfar, WSet &nxt, int hf, int s, int j) {
     const bool last = s + 1 == SPC;
-    if (j >= RT) af[j - RT] = last ? read_a(ci + 1, 0, j - RT) : read_a(ci, s + 1, j - RT);
-    if (s < 2 && j < 4) store_piece(r, ci + 1, 4 * s + j);
-    if (s < 2 && j >= 4 && j < 8) load_piece(r, ci + 3, 4 * s + j - 4);
+    if (j >= RT) af[j - RT] = last ? read_a(snxt, 0, j - RT) : read_a(scur, s + 1, j - RT);
+    if (s < 2 && j >= 4 && j < 8) load_piece(ci + 2, sfar, 4 * s + j - 4);
     if (s == 2 && hf == 0) {
       if (j < 8) load_w(nxt, (ci >> 1) + 1, j);
       if (j >= 8 && j - 8 < CT * NGRP) load_sz(nxt, (ci >> 1) + 1, j - 8);
     }
   };
-  auto chunk = [&](int ci, Staged &r, const WSet &cur, WSet &nxt, int hf) {
+  // Memory instructions issued after the activation loads of chunk ci + 1 when chunk ci reaches its barrier: this chunk's
+  // eight activation loads and one weight block's loads (issued in this chunk or the one before, whichever is a block's
+  // first half).  Loads complete in order, so that many may still be outstanding once chunk ci + 1 has landed.
+  constexpr int kLoadsBehind = kXPieces + 8 + CT * NGRP;
+  auto chunk = [&](int ci, uint32_t scur, uint32_t snxt, uint32_t sfar, const WSet &cur, WSet &nxt, int hf) {
 #pragma unroll
     for (int s = 0; s < SPC; ++s) {
       const int sa = 4 * hf + s;
-      if (s + 1 == SPC) lds_barrier();  // staging stores of this chunk visible, every wave done reading this stage
+      if (s + 1 == SPC)  // the next chunk has landed; behind the barrier every wave is done reading this stage
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kLoadsBehind) : "memory");
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) {
         // the operand to convert meanwhile: the next column tile's, or the first one of the following step
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
             if (nsa < 8) convert_part(cur, nct, nsa, rt >> 1);
             else convert_part(nxt, nct, 0, rt >> 1);
           }
-          slot_op(ci, r, nxt, hf, s, ct * RT + rt);
+          slot_op(ci, scur, snxt, sfar, nxt, hf, s, ct * RT + rt);
           __builtin_amdgcn_sched_barrier(0);
         }
         wf = __builtin_bit_cast(bf16x8_t, u32x4_t{cv[0], cv[1], cv[2], cv[3]});
@@ -188,35 +192,36 @@ __global__ __launch_bounds__(256) void int4_gemm128_kernel(const uint16_t *__res
     }
   };
 
-  Staged st[2];
   WSet ws[2];
 #pragma unroll
   for (int i = 0; i < 8; ++i) load_w(ws[0], 0, i);
 #pragma unroll
   for (int i = 0; i < CT * NGRP; ++i) load_sz(ws[0], 0, i);
 #pragma unroll
-  for (int i = 0; i < kXPieces; ++i) load_piece(st[0], 0, i);
+  for (int i = 0; i < kXPieces; ++i) load_piece(0, 0, i);
 #pragma unroll
-  for (int i = 0; i < kXPieces; ++i) store_piece(st[0], 0, i);
-#pragma unroll
-  for (int i = 0; i < kXPieces; ++i) load_piece(st[1], 1, i);
-#pragma unroll
-  for (int i = 0; i < kXPieces; ++i) load_piece(st[0], 2, i);
-  lds_barrier();
+  for (int i = 0; i < kXPieces; ++i) load_piece(1, kStageX, i);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kXPieces) : "memory");  // the weights of block 0 and chunk 0 are in
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) af[rt] = read_a(0, 0, rt);
 #pragma unroll
   for (int j = 0; j < 4; ++j) convert_part(ws[0], 0, 0, j);
   wf = __builtin_bit_cast(bf16x8_t, u32x4_t{cv[0], cv[1], cv[2], cv[3]});
-  for (int blk = 0; blk < nblocks; blk += 2) {  // two blocks per trip (K % 256 == 0): the register sets are compile-time names
-    chunk(2 * blk, st[1], ws[0], ws[1], 0);
-    chunk(2 * blk + 1, st[0], ws[0], ws[1], 1);
-    chunk(2 * blk + 2, st[1], ws[1], ws[0], 0);
-    chunk(2 * blk + 3, st[0], ws[1], ws[0], 1);
+  uint32_t s0 = 0, s1 = kStageX, s2 = 2 * kStageX;  // stage of the chunk in use, of the next one, of the one after
+  for (int blk = 0; blk < nblocks; blk += 2) {  // two blocks per trip (K % 256 == 0): the weight register sets are compile-time names
+    chunk(2 * blk, s0, s1, s2, ws[0], ws[1], 0);
+    chunk(2 * blk + 1, s1, s2, s0, ws[0], ws[1], 1);
+    chunk(2 * blk + 2, s2, s0, s1, ws[1], ws[0], 0);
+    chunk(2 * blk + 3, s0, s1, s2, ws[1], ws[0], 1);
+    const uint32_t t0 = s0;  // four chunks on: the rotation by three stages has advanced by one
+    s0 = s1;
+    s1 = s2;
+    s2 = t0;
   }
 
   // ---- store: lane (h, n) holds column col0 + 32 ct + n, rows 8 (e / 4) + 4 h + e % 4 of each tile -----------------
-  lds_barrier();  // the staging stages are dead from here on
+  // the loads issued past the last chunk still write LDS: drain them before the stages are reused
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   const float no_scale[CT] = {};
   store_tiles_via_lds<RT, CT, false>(acc, no_scale, lds + wave * TileStore<CT>::kBytesPerWave, y, row0, col0, M, N, lane,
                                     (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0);
