@@ -51,8 +51,8 @@ struct Options {
   int attention_no_mfma;   // 1 = grouped-query decode attention stays on the float32 vector kernel
   int int8_gemm_tile;      // 0 = heuristic, else 128 or 256 rows per workgroup in the many-row int8 matmul
   int int4_gemm_tile;      // 0 = heuristic, else 128 or 256 rows per workgroup in the many-row int4 matmul
-  int int8_gemm_waves;     // 0 or 4 = the 256-row workgroup is the four-wave kernel, 8 = the eight-wave one
-  int int8_gemm_wave_cols; // four-wave kernel: 0 or 4 = every wave 256 rows x 64 columns, 2 = 128 rows x 128 columns
+  int int8_gemm_waves;     // 256-row tiles: 0 = four waves fed by direct-to-LDS loads, 4 = four waves staging through registers, 8 = eight waves
+  int int8_gemm_wave_cols; // register-staged four-wave kernel: 0 or 4 = every wave 256 rows x 64 columns, 2 = 128 rows x 128 columns
   int staged_tiles;        // 0 = heuristic, else weight tiles per workgroup of the staged decode-batch int4 kernel
   int staged_slices;       // 0 = heuristic, else workgroups along K of that kernel (partial epilogue)
 };
