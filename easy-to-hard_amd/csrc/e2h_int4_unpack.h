@@ -85,7 +85,7 @@ __device__ __forceinline__ void store_tiles_via_lds(const e2h_f32x16_t (&acc)[CT
       if (row < M && col < N) {
         uint16_t *dst = y + static_cast<size_t>(row) * N + col;
         if (pieces) {
-          *reinterpret_cast<u32x4_t *>(dst) = v;
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t *>(dst));  // streamed: the tiles in L2 are the operands
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j)
