@@ -440,6 +440,32 @@ def test_int8_gemm32_tiles_match_oracle_and_16x16_kernel(m, n, k, tile, waves, w
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(2304, 8448, 128), (2304, 8448, 256), (4100, 4104, 384)])
+def test_int8_many_row_kernel_walks_several_tiles_per_workgroup(m, n, k):
+    """More 256 x 256 tiles than CUs, so that workgroups of the default many-row int8 kernel take a second tile while the
+    chunk pipeline runs on: the shortest K (two and four 64-wide chunks: the loads aimed two chunks ahead are already in
+    the next tile when a tile starts), a column-block count that leaves some XCDs a slot without a tile (33 and 17
+    blocks over 8 XCDs), ragged M and N.  Integer activations: every partial sum is an exact integer, so the result
+    must equal the reference's two-rounding form bit for bit and the 16x16-tile kernel's."""
+    q, s, q_d, s_d = _int8_case(n, k, seed=m + k)
+    xi = torch.randint(-2, 3, (m, k), generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    _lib.set_option("int8_gemm_tile", 256)
+    try:
+        yi = ops.int8_mm_direct(xi.to(DEV), q_d, s_d)
+    finally:
+        _lib.set_option("int8_gemm_tile", 0)
+    _lib.set_option("int4_no_gemm32", 1)
+    try:
+        yi2 = ops.int8_mm_direct(xi.to(DEV), q_d, s_d)
+    finally:
+        _lib.set_option("int4_no_gemm32", 0)
+    assert torch.equal(yi, yi2)
+    rows = np.r_[0:64, 255:258, m - 70:m]
+    y_rr = qo.int8_linear_reference_rounding(bf16_to_np(xi)[rows], q, s)
+    assert np.array_equal(bf16_to_np(yi)[rows], y_rr)
+
+
+@pytest.mark.gpu
 def test_int8_many_rows_at_the_reward_scoring_size():
     """One linear of the scoring configuration at its full row count (64 x 768 = 49152 rows, 4096 x 4096 weight):
     sampled rows against the oracle, row-permutation equivariance (a row's result does not depend on where in the
