@@ -15,7 +15,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_NAME = "libe2h_quant.so"
 LIB_PATH = PKG_DIR / LIB_NAME
 
-SOURCES = ["e2h_abi.hip", "e2h_quantize.hip", "e2h_int4_mm.hip", "e2h_int4_staged.hip", "e2h_int8_mm.hip", "e2h_int8_stream.hip", "e2h_int4_gemm.hip", "e2h_int4_gemm128.hip", "e2h_int8_gemm.hip", "e2h_attention.hip", "e2h_sample.hip", "e2h_probe.hip"]
+SOURCES = ["e2h_abi.hip", "e2h_quantize.hip", "e2h_int4_mm.hip", "e2h_int4_staged.hip", "e2h_int4_rows64.hip", "e2h_int8_mm.hip", "e2h_int8_stream.hip", "e2h_int4_gemm.hip", "e2h_int4_gemm128.hip", "e2h_int8_gemm.hip", "e2h_attention.hip", "e2h_sample.hip", "e2h_probe.hip"]
 
 # -ffp-contract=off: the quantizers are bit-exact restatements of separate torch ops; an FMA formed
 # across two of them would change codes.  packed-fp32-ops is switched off because some packed float32
@@ -35,7 +35,8 @@ HIPCC_FLAGS = [
 # Per-source additions.  The 32x32-tile matmul mixes MFMA accumulators with float32 FMAs on the same values; with
 # the accumulators in the accumulation register file every FMA needs copies in and out (3 extra instructions per FMA),
 # so that file is compiled with MFMA results kept in ordinary vector registers.
-EXTRA_FLAGS = {"e2h_int4_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "e2h_int4_staged.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}  # (the int8 kernel of the same shape has no such FMAs)
+EXTRA_FLAGS = {"e2h_int4_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "e2h_int4_staged.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+               "e2h_int4_rows64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}  # (the int8 kernel of the same shape has no such FMAs)
 
 
 def _hipcc():

@@ -113,6 +113,10 @@ extern "C" int e2h_set_option(const char *name, int value) {
     (name[7] == 't' ? o.staged_tiles : o.staged_slices) = value;
     return E2H_OK;
   }
+  if (!strcmp(name, "staged_no_rows64")) {
+    o.staged_no_rows64 = value != 0;
+    return E2H_OK;
+  }
   if (!strcmp(name, "attention_no_mfma")) {
     o.attention_no_mfma = value != 0;
     return E2H_OK;

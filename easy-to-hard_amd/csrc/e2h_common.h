@@ -55,6 +55,7 @@ struct Options {
   int int8_gemm_wave_cols; // register-staged four-wave kernel: 0 or 4 = every wave 256 rows x 64 columns, 2 = 128 rows x 128 columns
   int staged_tiles;        // 0 = heuristic, else weight tiles per workgroup of the staged decode-batch int4 kernel
   int staged_slices;       // 0 = heuristic, else workgroups along K of that kernel (partial epilogue)
+  int staged_no_rows64;    // 1 = 33 .. 64 rows with K-slice sums out stay on two 32-row slabs of the staged kernel
 };
 Options &options();
 

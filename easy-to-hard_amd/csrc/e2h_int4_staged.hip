@@ -545,6 +545,10 @@ extern "C" int e2h_int4_mm_staged(const void *staged, const int32_t *packed, con
 extern "C" int e2h_int4_mm_staged_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize) {
   const int rc = check_shape(m, n, k, groupsize);
   if (rc != E2H_OK) return rc;
+  if (m > 32 && !options().staged_no_rows64) {  // one pass over the weights for all rows
+    const int s64 = rows64_partial_slices(m, n, k, groupsize);
+    if (s64 > 0) return s64;
+  }
   StagedArgs a = {};
   Geometry g;
   if (!plan(&a, &g, nullptr, m, n, k, groupsize, kStPartial)) return E2H_ERR_BAD_SHAPE;
@@ -557,6 +561,8 @@ extern "C" int e2h_int4_mm_staged_partials(const void *staged, const int32_t *pa
   const int rc = check_shape(m, n, k, groupsize);
   if (rc != E2H_OK) return rc;
   if (!aligned16(staged) || !aligned16(packed) || !aligned16(scales_and_zeros) || (reinterpret_cast<uintptr_t>(partials) & 3u)) return E2H_ERR_MISALIGNED;
+  if (m > 32 && !options().staged_no_rows64 && rows64_partial_slices(m, n, k, groupsize) > 0)
+    return rows64_partials(staged, packed, scales_and_zeros, partials, m, n, k, groupsize, slices, static_cast<hipStream_t>(stream));
   StagedArgs a = {};
   Geometry g;
   if (!plan(&a, &g, staged, m, n, k, groupsize, kStPartial)) return E2H_ERR_BAD_SHAPE;

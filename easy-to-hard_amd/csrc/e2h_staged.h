@@ -33,6 +33,12 @@ inline StagedOut staged_out(void *buf, int64_t m, int64_t k) {
   return o;
 }
 
+// 33 .. 64 rows, K-slice sums out, one pass over the weights (e2h_int4_rows64.hip): number of slices (0: not covered)
+// and the launch; same arguments and result layout as the partial-sum entry point of e2h_int4_staged.hip.
+int rows64_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize);
+int rows64_partials(const void *staged, const int32_t *packed, const uint16_t *sz, float *partials, int64_t m, int64_t n, int64_t k,
+                    int groupsize, int slices, hipStream_t stream);
+
 #if defined(__HIPCC__)
 // Eight consecutive values of row m (16-byte piece number pc of the row, raw = four dwords of two bfloat16 each).  The
 // two lanes that hold pieces 2i and 2i + 1 of a row must be neighbours (lane ^ 1) and must both call.

@@ -29,7 +29,7 @@ FUSE_ROPE_PROJECTION = True  # q|k|v projection + RoPE + cache write as one int4
 DEFER_SPLIT_K = True         # wo / w2 hand float32 K-slice sums to the residual add + RMSNorm instead of combining them
 STAGED_DECODE = True         # int4 decode step: activations travel between the kernels in matrix-core operand order
 STAGED_HEAD = True           # ... including the LM head
-STAGED_MAX_ROWS = 32         # beyond one 32-row slab the row-major kernels are as fast or faster (34B shapes at 64 rows)
+STAGED_MAX_ROWS = 64         # 33 .. 64 rows: wo and w2 run the one-pass 64-row kernel, the other launches two 32-row slabs
 
 
 def _fusable(t: Tensor) -> bool:

@@ -42,7 +42,7 @@ const char *e2h_status_string(int status);
 /* Tuning knobs for experiments: launch-geometry overrides such as "int4_rows_per_wave", "int4_k_slices", "int4_k_groups",
  * "int4_col_waves", "int8_rows_per_wave", "int8_k_groups", "int8_k_slices", "int8_force_generic", "row_tiles", "int4_no_xsum",
  * "int4_no_gemm32", "int4_gemm32_min_rows", "int4_gemm_tile", "int8_gemm_tile", "int8_gemm_waves", "int8_gemm_wave_cols", "attention_waves",
- * "attention_no_mfma", "staged_tiles", "staged_slices";
+ * "attention_no_mfma", "staged_tiles", "staged_slices", "staged_no_rows64";
  * value 0 restores the built-in heuristic.  Not thread safe; set before launching. */
 int e2h_set_option(const char *name, int value);
 
@@ -279,7 +279,8 @@ int e2h_int4_mm_staged(const void *staged, const int32_t *packed, const uint16_t
 /* The same product left as float32 sums over `slices` contiguous parts of K, partials [slices, m, n], for
  * e2h_add_rmsnorm_staged to add in slice order (the wo / w2 projections of a decoder block, reference
  * models/model.py:279-283).  e2h_int4_mm_staged_partial_slices returns the library's slice count for the shape (>= 1) or
- * a negative status; any other `slices` is rejected. */
+ * a negative status; any other `slices` is rejected.  (33 .. 64 rows run a kernel of their own that covers all rows in
+ * one pass over the weights; same arguments, same layout of the result.) */
 int e2h_int4_mm_staged_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize);
 int e2h_int4_mm_staged_partials(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, float *partials,
                                 int64_t m, int64_t n, int64_t k, int groupsize, int slices, void *stream);
