@@ -361,3 +361,29 @@ def test_staged_decode_step_agrees_with_the_row_major_fused_step(monkeypatch):
         first = torch.argmax(logits[True][0], dim=-1, keepdim=True)
         tok = stepper.step(first, torch.tensor([t + 1], device=DEV)).clone()
         assert torch.equal(tok, torch.argmax(logits[True][1], dim=-1, keepdim=True))
+
+
+@pytest.mark.gpu
+def test_read_only_probe_accepts_and_rejects_as_declared():
+    """e2h_stream_read_probe (the launch behind `bench.py --floor`): it writes nothing, so what can be checked is that
+    the documented argument ranges are accepted (empty launch, private bytes only, private + shared) and that bad sizes,
+    a missing pointer and a misaligned one come back as their status codes."""
+    import ctypes
+
+    from easy_to_hard_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+    shared = torch.zeros(1 << 16, dtype=torch.uint8, device=DEV)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p, s = ctypes.c_void_p(buf.data_ptr()), ctypes.c_void_p(shared.data_ptr())
+    assert lib.e2h_stream_read_probe(None, 0, None, 0, None, stream) == 0
+    assert lib.e2h_stream_read_probe(p, buf.numel(), None, 0, None, stream) == 0
+    assert lib.e2h_stream_read_probe(p, buf.numel(), s, shared.numel(), None, stream) == 0
+    assert lib.e2h_stream_read_probe(p, 24, None, 0, None, stream) == -2          # not a multiple of 16
+    assert lib.e2h_stream_read_probe(p, 1 << 31, None, 0, None, stream) == -2     # beyond the 2 GB a launch addresses
+    assert lib.e2h_stream_read_probe(None, 16, None, 0, None, stream) == -1
+    assert lib.e2h_stream_read_probe(p, 16, None, 16, None, stream) == -1
+    assert lib.e2h_stream_read_probe(ctypes.c_void_p(buf.data_ptr() + 8), 16, None, 0, None, stream) == -5
+    torch.cuda.synchronize()
+    assert not buf.any() and not shared.any()
