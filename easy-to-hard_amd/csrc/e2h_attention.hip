@@ -240,10 +240,11 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
   for (int nt = 0; nt < 8; ++nt) oacc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   for (int t0 = wave * 32; t0 < n_live; t0 += NW * 32) {
-    // K operands of the two 16-position halves and this lane's share of the V tile (row = lane / 2 + 32-row wrap,
-    // eight 16-byte pieces of its half row), all requested before anything is waited for.  Default cache policy: a K row
-    // is covered by four instructions and a V row by eight, and with streaming loads (which pay off in the kernel above,
-    // whose every instruction covers whole rows) the pieces of a line are fetched again and again: 1.7 x the time.
+    // K operands of the two 16-position halves and this lane's share of the V tile (eight 16-byte pieces: piece
+    // lane % 16 of rows lane / 16 + 4 i), all requested before anything is waited for.  The V loads cover whole rows per
+    // instruction and stream (8 % less time than with the default policy); a K row is covered by four instructions in
+    // operand order, and streamed that way the pieces of a line are fetched again and again (1.7 x the time), so the K
+    // loads keep the default policy.
     u32x4_t kf[2][4], vr[8];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -252,12 +253,11 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) kf[j][s4] = *reinterpret_cast<const u32x4_t *>(kbase + static_cast<size_t>(tc) * D + 32 * s4);
     }
-    {
-      const int vrow = lane >> 1, vhalf = lane & 1;
-      const int tp = t0 + vrow;
-      const int tc = tp < n_live ? tp : n_live - 1;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) vr[i] = *reinterpret_cast<const u32x4_t *>(vbase + static_cast<size_t>(tc) * D + 64 * vhalf + 8 * i);
+    for (int i = 0; i < 8; ++i) {  // instruction i: rows 4 i .. 4 i + 3 of the tile, sixteen lanes per 256-byte row
+      const int tp = t0 + 4 * i + (lane >> 4);
+      const int tc = tp < n_live ? tp : n_live - 1;
+      vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(vbase + static_cast<size_t>(tc) * D + 8 * (lane & 15)));
     }
     // S = Q K^T for 32 positions
     f32x4_t sacc[2];
@@ -270,12 +270,11 @@ __global__ __launch_bounds__(64 * NW) void decode_attention_gqa_kernel(const uin
     }
     // the V tile goes to LDS while the softmax is worked out
     {
-      const int vrow = lane >> 1, vhalf = lane & 1;
-      uint8_t *dst = v_lds + vrow * kGqaVRow + 128 * vhalf;
+      uint8_t *dst = v_lds + (lane >> 4) * kGqaVRow + 16 * (lane & 15);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        *reinterpret_cast<u32x2_t *>(dst + 16 * i) = u32x2_t{vr[i][0], vr[i][1]};
-        *reinterpret_cast<u32x2_t *>(dst + 16 * i + 8) = u32x2_t{vr[i][2], vr[i][3]};
+        *reinterpret_cast<u32x2_t *>(dst + 4 * i * kGqaVRow) = u32x2_t{vr[i][0], vr[i][1]};
+        *reinterpret_cast<u32x2_t *>(dst + 4 * i * kGqaVRow + 8) = u32x2_t{vr[i][2], vr[i][3]};
       }
     }
     float pv[2][4], corr[4];
