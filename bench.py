@@ -585,6 +585,8 @@ def main():
         pos = torch.tensor([t_prompt], device=dev, dtype=torch.int64)
         for _ in range(args.warmup):
             stepper.step(cur, pos)
+            pos += 1  # also loads the kernel of this update, whose first use costs tens of milliseconds
+        pos.fill_(t_prompt)
         cur = prefill(model, prompt, input_pos)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
