@@ -67,7 +67,7 @@ def parse_args():
                          "linear goes through PyTorch-ROCm's aten._weight_int4pack_mm and everything around the linears through "
                          "stock torch ops (what the reference's model code executes, without inductor); prints its own JSON line")
     ap.add_argument("--model-switch", action="append", default=[], metavar="NAME=0|1",
-                    help="set a fusion switch of easy_to_hard_amd.model (FUSE_GATE, FUSE_ROPE_PROJECTION, DEFER_SPLIT_K, STAGED_DECODE, STAGED_HEAD) for a comparison run")
+                    help="set a fusion switch of easy_to_hard_amd.model (FUSE_GATE, FUSE_ROPE_PROJECTION, DEFER_SPLIT_K, STAGED_DECODE, STAGED_HEAD, FUSE_HEAD_ARGMAX) for a comparison run")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch-geometry override passed to e2h_set_option (experiments)")
     ap.add_argument("--full-decode", action="store_true",
@@ -506,7 +506,7 @@ def main():
         import easy_to_hard_amd.model as model_mod
 
         name, _, value = item.partition("=")
-        assert name in ("FUSE_GATE", "FUSE_ROPE_PROJECTION", "DEFER_SPLIT_K", "STAGED_DECODE", "STAGED_HEAD"), name
+        assert name in ("FUSE_GATE", "FUSE_ROPE_PROJECTION", "DEFER_SPLIT_K", "STAGED_DECODE", "STAGED_HEAD", "FUSE_HEAD_ARGMAX"), name
         setattr(model_mod, name, bool(int(value)))
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda", 0)

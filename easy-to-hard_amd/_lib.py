@@ -50,6 +50,8 @@ _SIGNATURES = {
     "e2h_int4_stage_x": (c_int, [_P, _P, c_int64, c_int64, _P]),
     "e2h_int4_mm_staged_supported": (c_int, [c_int64, c_int64, c_int64, c_int, c_int]),
     "e2h_int4_mm_staged": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),
+    "e2h_int4_mm_staged_argmax_scratch_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int]),
+    "e2h_int4_mm_staged_argmax": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),
     "e2h_int4_mm_staged_partial_slices": (c_int, [c_int64, c_int64, c_int64, c_int]),
     "e2h_int4_mm_staged_partials": (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, c_int, _P]),
     "e2h_int4_mm_staged_silu_gate": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int, _P]),

@@ -240,6 +240,13 @@ def _mm_staged(buf: Tensor, rows: int, k: int, packed: Tensor, groupsize: int, s
     return _mm_staged_eager(_as_eager(buf, rows, k), packed, groupsize, scales_and_zeros)
 
 
+_mm_staged_argmax_eager = _ops.int4_mm_staged_argmax
+
+
+def _mm_staged_argmax(buf: Tensor, rows: int, k: int, packed: Tensor, groupsize: int, scales_and_zeros: Tensor) -> Tensor:
+    return _mm_staged_argmax_eager(_as_eager(buf, rows, k), packed, groupsize, scales_and_zeros)
+
+
 _mm_staged_partials_eager = _ops.int4_mm_staged_partials
 
 
@@ -287,6 +294,8 @@ def _u8(t, n):
 
 _stage_x_op = _register("int4_stage_x", _stage_x, lambda x: _u8(x, _staged_bytes(x.shape[0], x.shape[1])))
 _mm_staged_op = _register("int4_mm_staged", _mm_staged, lambda buf, rows, k, p, g, sz: _like(sz, (rows, p.shape[0] * 8)))
+_mm_staged_argmax_op = _register("int4_mm_staged_argmax", _mm_staged_argmax,
+                                 lambda buf, rows, k, p, g, sz: _like(sz, (rows, 1), torch.int64))
 _mm_staged_partials_op = _register("int4_mm_staged_partials", _mm_staged_partials,
                                    lambda buf, rows, k, p, g, sz, s: _like(sz, (s, rows, p.shape[0] * 8), torch.float32))
 _mm_staged_gate_op = _register(
@@ -313,6 +322,11 @@ def stage_x(x):
 def int4_mm_staged(xs, packed, groupsize, scales_and_zeros):
     """int4_mm on staged activations -> bf16 [rows, N]."""
     return _mm_staged_op(xs.buf, xs.rows, xs.k, packed, groupsize, scales_and_zeros)
+
+
+def int4_mm_staged_argmax(xs, packed, groupsize, scales_and_zeros):
+    """argmax over the columns of int4_mm_staged(xs, ...) without storing the product -> int64 [rows, 1]."""
+    return _mm_staged_argmax_op(xs.buf, xs.rows, xs.k, packed, groupsize, scales_and_zeros)
 
 
 def int4_mm_staged_partials(xs, packed, groupsize, scales_and_zeros, slices):
@@ -415,7 +429,7 @@ def int4_staged_partial_slices(rows, lin):
 _REBOUND = (
     "rmsnorm", "add_rmsnorm", "silu_mul", "rope_kv_write", "rope_kv_write_seq", "decode_attention", "argmax_rows", "int4_mm_silu_gate",
     "int4_mm_rope_kv", "int4_mm_partials", "int8_mm_silu_gate", "int8_mm_rope_kv", "int8_mm_partials", "ScaledPartials",
-    "StagedActivations", "stage_x", "int4_mm_staged", "int4_mm_staged_partials", "int4_mm_staged_silu_gate", "int4_mm_staged_rope_kv",
+    "StagedActivations", "stage_x", "int4_mm_staged", "int4_mm_staged_argmax", "int4_mm_staged_partials", "int4_mm_staged_silu_gate", "int4_mm_staged_rope_kv",
     "add_rmsnorm_staged", "decode_attention_staged", "int8_quantize_per_channel", "int4_group_quantize", "int4_unpack",
     "int4_partial_slices", "int8_partial_slices", "int4_staged_supported", "int4_staged_partial_slices",
 )

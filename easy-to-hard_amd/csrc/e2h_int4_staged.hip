@@ -35,7 +35,7 @@ constexpr int kWaves = 8;
 constexpr int kNt = 2;  // "nt" cache policy: weights are streamed once
 constexpr int kCUs = 256;
 
-enum StagedEpilogue { kStPlain = 0, kStGate = 1, kStRope = 2, kStPartial = 3 };
+enum StagedEpilogue { kStPlain = 0, kStGate = 1, kStRope = 2, kStPartial = 3, kStArgmax = 4 };
 
 struct StagedRope {
   const uint16_t *freqs;     // [>= S, D/2, 2] bf16 (cos, sin)
@@ -50,6 +50,7 @@ struct StagedArgs {
   const uint32_t *wp, *sz, *wp2, *sz2;
   uint16_t *y;          // bf16 [M][N] (plain, gate; may be null for gate when only the staged result is wanted)
   float *partials;      // f32 [S][M][N] (partial)
+  unsigned long long *cand;  // [column blocks][M] (arg-max): per row the best (value key << 32 | ~column) of the block's columns
   StagedOut out;        // gate: the result in staged form for the next linear (frag null: not wanted)
   int M, Mpad, N, K;
   int slabs, col_blocks;
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(64 * kWaves) void int4_staged_mm_kernel(const Stage
   constexpr int kAccFloats = T * MT * 4 * 64;
 
   __shared__ __attribute__((aligned(16))) float red[kWaves * kAccFloats];
+  __shared__ unsigned long long unit_best[EPI == kStArgmax ? kUnits : 1][16];  // arg-max: per unit and row of its tile
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -369,6 +371,23 @@ __global__ __launch_bounds__(64 * kWaves) void int4_staged_mm_kernel(const Stage
         const float r = (c & 1) ? own * cs + other * sn : own * cs - other * sn;
         if (in_range && m < M) dst[static_cast<size_t>(m) * row_stride] = f32_to_bf16_rne(rotated ? r : own);
       }
+    } else if constexpr (EPI == kStArgmax) {
+      // greedy token straight from the LM head: the logit is rounded to bfloat16 as the plain epilogue would store it and
+      // offered as (order-preserving key << 32 | ~column), so that the maximum is the largest value and, among equals,
+      // the lowest column; a NaN counts as the largest value (torch.argmax over the float32 view of bfloat16 logits,
+      // reference inference_generate.py:110-120 with sampling switched off).  First over the tile's 16 columns ...
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t u = static_cast<uint32_t>(f32_to_bf16_rne(v[0][q])) << 16;
+        const uint32_t key = (u & 0x7FFFFFFFu) > 0x7F800000u ? 0xFFFFFFFFu : ((u & 0x80000000u) ? ~u : (u | 0x80000000u));
+        unsigned long long best = n < N ? ((static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(~static_cast<uint32_t>(n))) : 0ull;
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+          const unsigned long long other = __shfl_xor(best, off);
+          best = other > best ? other : best;
+        }
+        if (c == 0) unit_best[unit][4 * b + q] = best;
+      }
     } else {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -377,6 +396,33 @@ __global__ __launch_bounds__(64 * kWaves) void int4_staged_mm_kernel(const Stage
       }
     }
   }
+  if constexpr (EPI == kStArgmax) {
+    // ... then over the workgroup's column tiles: one candidate per row and column block for the reduction kernel
+    __syncthreads();
+    if (tid < 16 * MT) {
+      const int mt = tid >> 4, m = m_base + tid;
+      unsigned long long best = 0ull;
+#pragma unroll
+      for (int tc = 0; tc < TC; ++tc) best = unit_best[tc * MT + mt][tid & 15] > best ? unit_best[tc * MT + mt][tid & 15] : best;
+      if (m < M) a.cand[static_cast<size_t>(col_block) * M + m] = best;
+    }
+  }
+}
+
+// arg-max: the candidates of all column blocks of a row -> the row's token (one wave per row)
+__global__ __launch_bounds__(64) void argmax_candidates_kernel(const unsigned long long *__restrict__ cand, int blocks, int M, int64_t *__restrict__ out) {
+  const int m = blockIdx.x;
+  unsigned long long best = 0ull;
+  for (int i = threadIdx.x; i < blocks; i += 64) {
+    const unsigned long long v = cand[static_cast<size_t>(i) * M + m];
+    best = v > best ? v : best;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned long long other = __shfl_xor(best, off);
+    best = other > best ? other : best;
+  }
+  if (threadIdx.x == 0) out[m] = static_cast<int64_t>(~static_cast<uint32_t>(best & 0xFFFFFFFFull));
 }
 
 // ---- staging pass: row-major activations -> operand order + sums of 16 ------------------------------------------------
@@ -402,6 +448,7 @@ struct Inst {
   int t, c, dw, dx;
 };
 constexpr Inst kPlainInsts[] = {{3, 4, 2, 2}, {4, 4, 2, 2}, {8, 4, 1, 1}, {6, 4, 2, 1}, {2, 2, 2, 2}, {4, 2, 2, 2}, {6, 2, 2, 2}, {4, 1, 1, 1}, {4, 3, 3, 1}, {4, 8, 2, 1}, {8, 8, 1, 1}, {2, 1, 1, 1}};
+constexpr Inst kArgmaxInsts[] = {{8, 4, 1, 1}, {4, 4, 2, 2}, {8, 8, 1, 1}, {4, 8, 2, 1}, {4, 1, 1, 1}, {2, 1, 1, 1}};  // LM heads: few K shapes
 constexpr Inst kGateInsts[] = {{6, 4, 2, 1}, {4, 4, 2, 2}, {8, 4, 1, 1}, {6, 8, 1, 1}, {8, 8, 1, 1}};
 
 // instantiations that do not fit the 256 vector registers of a wave (they would run, slowly, out of scratch memory):
@@ -452,6 +499,8 @@ int dispatch_inst(const StagedArgs &a, const Geometry &g, hipStream_t stream) {
   if (g.t == TV && g.c == CV && g.dw == DWV && g.dx == DXV) return launch_staged<G, MT, TV, CV, DWV, DXV, EPI>(a, g.slices, stream);
   if constexpr (EPI == kStGate) {
     E2H_ST_CASE(6, 4, 2, 1) E2H_ST_CASE(4, 4, 2, 2) E2H_ST_CASE(8, 4, 1, 1) E2H_ST_CASE(6, 8, 1, 1) E2H_ST_CASE(8, 8, 1, 1)
+  } else if constexpr (EPI == kStArgmax) {
+    E2H_ST_CASE(8, 4, 1, 1) E2H_ST_CASE(4, 4, 2, 2) E2H_ST_CASE(8, 8, 1, 1) E2H_ST_CASE(4, 8, 2, 1) E2H_ST_CASE(4, 1, 1, 1) E2H_ST_CASE(2, 1, 1, 1)
   } else {
     E2H_ST_CASE(3, 4, 2, 2) E2H_ST_CASE(4, 4, 2, 2) E2H_ST_CASE(8, 4, 1, 1) E2H_ST_CASE(6, 4, 2, 1) E2H_ST_CASE(2, 2, 2, 2)
     E2H_ST_CASE(4, 2, 2, 2) E2H_ST_CASE(6, 2, 2, 2) E2H_ST_CASE(4, 1, 1, 1) E2H_ST_CASE(2, 1, 1, 1) E2H_ST_CASE(4, 3, 3, 1) E2H_ST_CASE(4, 8, 2, 1) E2H_ST_CASE(8, 8, 1, 1)
@@ -492,6 +541,7 @@ bool plan(StagedArgs *a, Geometry *g, const void *staged, int64_t m, int64_t n, 
   const int kt = static_cast<int>(k / 128);
   bool ok;
   if (epi == kStGate) ok = pick(kGateInsts, true, groupsize, tiles16, kt, a->slabs, 1, g);
+  else if (epi == kStArgmax) ok = pick(kArgmaxInsts, false, groupsize, tiles16, kt, a->slabs, 1, g);
   else ok = pick(kPlainInsts, false, groupsize, tiles16, kt, a->slabs, epi == kStPartial ? 8 : 1, g);
   if (!ok) return false;
   const int tc = epi == kStGate ? g->t / 2 : g->t;
@@ -521,7 +571,7 @@ extern "C" int e2h_int4_stage_x(const uint16_t *x, void *staged, int64_t m, int6
 }
 
 extern "C" int e2h_int4_mm_staged_supported(int64_t m, int64_t n, int64_t k, int groupsize, int epilogue) {
-  if (check_shape(m, n, k, groupsize) != E2H_OK || epilogue < 0 || epilogue > 3) return 0;
+  if (check_shape(m, n, k, groupsize) != E2H_OK || epilogue < 0 || epilogue > 4) return 0;
   StagedArgs a = {};
   Geometry g;
   return plan(&a, &g, nullptr, m, n, k, groupsize, epilogue) ? 1 : 0;
@@ -540,6 +590,36 @@ extern "C" int e2h_int4_mm_staged(const void *staged, const int32_t *packed, con
   a.sz = reinterpret_cast<const uint32_t *>(scales_and_zeros);
   a.y = y;
   return dispatch_staged<kStPlain>(a, groupsize, g, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t e2h_int4_mm_staged_argmax_scratch_bytes(int64_t m, int64_t n, int64_t k, int groupsize) {
+  const int rc = check_shape(m, n, k, groupsize);
+  if (rc != E2H_OK) return rc;
+  StagedArgs a = {};
+  Geometry g;
+  if (!plan(&a, &g, nullptr, m, n, k, groupsize, kStArgmax)) return E2H_ERR_BAD_SHAPE;
+  return static_cast<int64_t>(a.col_blocks) * m * 8;
+}
+
+extern "C" int e2h_int4_mm_staged_argmax(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, void *scratch,
+                                         int64_t *tokens, int64_t m, int64_t n, int64_t k, int groupsize, void *stream) {
+  if (!staged || !packed || !scales_and_zeros || !scratch || !tokens) return E2H_ERR_NULL_POINTER;
+  const int rc = check_shape(m, n, k, groupsize);
+  if (rc != E2H_OK) return rc;
+  if (!aligned16(staged) || !aligned16(packed) || !aligned16(scales_and_zeros) || (reinterpret_cast<uintptr_t>(scratch) & 7u) ||
+      (reinterpret_cast<uintptr_t>(tokens) & 7u))
+    return E2H_ERR_MISALIGNED;
+  StagedArgs a = {};
+  Geometry g;
+  if (!plan(&a, &g, staged, m, n, k, groupsize, kStArgmax)) return E2H_ERR_BAD_SHAPE;
+  a.wp = reinterpret_cast<const uint32_t *>(packed);
+  a.sz = reinterpret_cast<const uint32_t *>(scales_and_zeros);
+  a.cand = static_cast<unsigned long long *>(scratch);
+  const int rc2 = dispatch_staged<kStArgmax>(a, groupsize, g, static_cast<hipStream_t>(stream));
+  if (rc2 != E2H_OK) return rc2;
+  hipLaunchKernelGGL(argmax_candidates_kernel, dim3(static_cast<unsigned>(m)), dim3(64), 0, static_cast<hipStream_t>(stream), a.cand,
+                     a.col_blocks, a.M, tokens);
+  return launch_status();
 }
 
 extern "C" int e2h_int4_mm_staged_partial_slices(int64_t m, int64_t n, int64_t k, int groupsize) {

@@ -58,6 +58,14 @@ def _next_token(logits: Tensor, temperature: Optional[float], top_k: Optional[in
     return sample(logits, temperature, top_k)[0].to(torch.int64)
 
 
+def _greedy_through_the_model(model) -> bool:
+    """True for this package's Transformer, whose forward can return the greedy token itself (a wrapped or compiled
+    module, or a stand-in with the reference's signature, is asked for logits)."""
+    from .model import Transformer
+
+    return isinstance(model, Transformer)
+
+
 @torch.no_grad()
 def prefill(model, x: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None,
             temperature: Optional[float] = None, top_k: Optional[int] = None) -> Tensor:
@@ -69,6 +77,8 @@ def prefill(model, x: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Ten
 def decode_one_token(model, cur_token: Tensor, input_pos: Tensor, left_pad_mask_pos: Optional[Tensor] = None,
                      temperature: Optional[float] = None, top_k: Optional[int] = None) -> Tensor:
     assert input_pos.shape[-1] == 1
+    if temperature is None and _greedy_through_the_model(model):
+        return model(cur_token, input_pos, left_pad_mask_pos, greedy_token=True)
     return _next_token(model(cur_token, input_pos, left_pad_mask_pos), temperature, top_k)
 
 

@@ -29,6 +29,7 @@ FUSE_ROPE_PROJECTION = True  # q|k|v projection + RoPE + cache write as one int4
 DEFER_SPLIT_K = True         # wo / w2 hand float32 K-slice sums to the residual add + RMSNorm instead of combining them
 STAGED_DECODE = True         # int4 decode step: activations travel between the kernels in matrix-core operand order
 STAGED_HEAD = True           # ... including the LM head
+FUSE_HEAD_ARGMAX = True      # greedy decoding: the LM head launch reduces its columns to the arg-max, no logits are stored
 STAGED_MAX_ROWS = 64         # 33 .. 64 rows: wo and w2 run the one-pass 64-row kernel, the other launches two 32-row slabs
 
 
@@ -405,8 +406,23 @@ class Transformer(nn.Module):
         return all(_staged_block_supported(blk, rows) for blk in self.layers)
 
     def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None, left_pad_mask_pos: Optional[Tensor] = None,
-                fully_causal: bool = False) -> Tensor:
-        """idx [B, S] token ids, input_pos [S] positions -> logits [B, S, vocab] (reference :212-248)."""
+                fully_causal: bool = False, greedy_token: bool = False) -> Tensor:
+        """idx [B, S] token ids, input_pos [S] positions -> logits [B, S, vocab] (reference :212-248).
+
+        greedy_token=True (not in the reference's signature; what its decode loop computes from the logits with sampling
+        switched off, inference_generate.py:110-120): -> int64 [B, 1], argmax over the vocabulary of the last position's
+        logits.  In the single-token step of an int4 model the LM head launch itself reduces its columns, so the
+        logits are never stored."""
+        logits = self._forward(idx, input_pos, left_pad_mask_pos, fully_causal, greedy_token)
+        if not greedy_token or logits.dtype == torch.int64:
+            return logits
+        last = logits[:, -1]
+        if last.is_cuda and last.dtype == torch.bfloat16:
+            return ops.argmax_rows(last)
+        return torch.argmax(last.float(), dim=-1, keepdim=True)
+
+    def _forward(self, idx: Tensor, input_pos: Optional[Tensor], left_pad_mask_pos: Optional[Tensor], fully_causal: bool,
+                 greedy_token: bool) -> Tensor:
         assert self.freqs_cis is not None, "Caches must be initialized first"
         assert not (fully_causal and left_pad_mask_pos is not None), "Invalid mask"
         for blk in self.layers:
@@ -433,6 +449,8 @@ class Transformer(nn.Module):
             out = self.output
             if isinstance(out, WeightOnlyInt4Linear) and STAGED_HEAD and ops.int4_staged_supported(rows, out, ops.STAGED_PLAIN):
                 _, _, xs = ops.add_rmsnorm_staged(h, delta, self.norm.weight, self.norm.eps)
+                if greedy_token and FUSE_HEAD_ARGMAX and ops.int4_staged_supported(rows, out, ops.STAGED_ARGMAX):
+                    return ops.int4_mm_staged_argmax(xs, out.weight, out.groupsize, out.scales_and_zeros)
                 return ops.int4_mm_staged(xs, out.weight, out.groupsize, out.scales_and_zeros).view(rows, 1, -1)
             _, normed = ops.add_rmsnorm(h, delta, self.norm.weight, self.norm.eps)
             return self.output(normed.view(rows, 1, -1))

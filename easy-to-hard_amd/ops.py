@@ -680,7 +680,7 @@ def decode_attention(q, k_cache, v_cache, input_pos, left_pad_mask_pos=None, sca
 # by stage_x for activations that arrive row-major
 # ---------------------------------------------------------------------------------------------
 
-STAGED_PLAIN, STAGED_GATE, STAGED_ROPE, STAGED_PARTIAL = 0, 1, 2, 3
+STAGED_PLAIN, STAGED_GATE, STAGED_ROPE, STAGED_PARTIAL, STAGED_ARGMAX = 0, 1, 2, 3, 4
 
 
 class StagedActivations:
@@ -739,6 +739,23 @@ def int4_mm_staged(xs, packed, groupsize, scales_and_zeros):
     rc = _lib_for(y).e2h_int4_mm_staged(_ptr(xs.buf), _ptr(packed), _ptr(scales_and_zeros), _ptr(y), xs.rows, n, k, groupsize, _stream(y))
     _lib.check(rc, "e2h_int4_mm_staged")
     return y
+
+
+def int4_mm_staged_argmax(xs, packed, groupsize, scales_and_zeros):
+    """argmax over the columns of int4_mm_staged(xs, ...) without storing the product -> int64 [rows, 1] (greedy token from
+    the LM head; lowest index among ties, a NaN counts as the maximum, as argmax_rows)."""
+    _need_gpu(xs.buf, packed, scales_and_zeros)
+    n, k = _staged_dims(xs, packed, scales_and_zeros, groupsize, "int4_mm_staged_argmax")
+    lib = _lib_for(xs.buf)
+    nbytes = int(lib.e2h_int4_mm_staged_argmax_scratch_bytes(xs.rows, n, k, groupsize))
+    if nbytes <= 0:
+        _lib.check(nbytes if nbytes < 0 else -2, "e2h_int4_mm_staged_argmax_scratch_bytes")
+    scratch = torch.empty((nbytes // 8,), dtype=torch.int64, device=xs.device)
+    tokens = torch.empty((xs.rows, 1), dtype=torch.int64, device=xs.device)
+    rc = lib.e2h_int4_mm_staged_argmax(_ptr(xs.buf), _ptr(packed), _ptr(scales_and_zeros), _ptr(scratch), _ptr(tokens), xs.rows, n, k,
+                                       groupsize, _stream(tokens))
+    _lib.check(rc, "e2h_int4_mm_staged_argmax")
+    return tokens
 
 
 def int4_staged_partial_slices(rows, lin):

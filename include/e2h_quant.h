@@ -269,12 +269,23 @@ int64_t e2h_int4_staged_bytes(int64_t m, int64_t k);
 int e2h_int4_stage_x(const uint16_t *x, void *staged, int64_t m, int64_t k, void *stream);
 
 /* 1 if a staged decode-batch kernel exists for the shape and epilogue (0 = e2h_int4_mm_staged, 1 = _silu_gate,
- * 2 = _rope_kv, 3 = _partials), else 0. */
+ * 2 = _rope_kv, 3 = _partials, 4 = _argmax), else 0. */
 int e2h_int4_mm_staged_supported(int64_t m, int64_t n, int64_t k, int groupsize, int epilogue);
 
 /* linear_forward_int4, reference :445-453: y [m, n] bf16 = staged x times the packed weight. */
 int e2h_int4_mm_staged(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, uint16_t *y, int64_t m,
                        int64_t n, int64_t k, int groupsize, void *stream);
+
+/* Greedy next token straight from the LM head (reference inference_generate.py:110-120 with sampling switched off:
+ * torch.argmax over the logits of the last position; models/model.py:247 is the head): tokens[r] = argmax_n of
+ * bf16(staged x times the packed weight)[r, n] without the logits ever being stored -- every workgroup of the matmul
+ * reduces its columns to one candidate per row, a second small launch picks each row's best.  The same answer as
+ * e2h_argmax_rows over e2h_int4_mm_staged's result (lowest index among ties, a NaN counts as the maximum).
+ *   scratch: e2h_int4_mm_staged_argmax_scratch_bytes(m, n, k, groupsize) bytes (or a negative status), 8-byte aligned,
+ *   overwritten; tokens int64 [m]. */
+int64_t e2h_int4_mm_staged_argmax_scratch_bytes(int64_t m, int64_t n, int64_t k, int groupsize);
+int e2h_int4_mm_staged_argmax(const void *staged, const int32_t *packed, const uint16_t *scales_and_zeros, void *scratch,
+                              int64_t *tokens, int64_t m, int64_t n, int64_t k, int groupsize, void *stream);
 
 /* The same product left as float32 sums over `slices` contiguous parts of K, partials [slices, m, n], for
  * e2h_add_rmsnorm_staged to add in slice order (the wo / w2 projections of a decoder block, reference

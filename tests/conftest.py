@@ -34,7 +34,7 @@ _LIBRARY_OPTIONS = (
     "int8_force_generic", "int8_k_slices", "int4_no_xsum", "int4_no_gemm32", "int4_gemm32_min_rows", "row_tiles",
     "attention_waves", "int8_gemm_waves", "int8_gemm_wave_cols", "int4_gemm_tile", "int8_gemm_tile", "attention_no_mfma", "staged_tiles", "staged_slices", "staged_no_rows64",
 )
-_MODEL_SWITCHES = ("FUSED_DECODE", "FUSE_GATE", "FUSE_ROPE_PROJECTION", "DEFER_SPLIT_K", "STAGED_DECODE", "STAGED_HEAD")
+_MODEL_SWITCHES = ("FUSED_DECODE", "FUSE_GATE", "FUSE_ROPE_PROJECTION", "DEFER_SPLIT_K", "STAGED_DECODE", "STAGED_HEAD", "FUSE_HEAD_ARGMAX")
 
 
 @pytest.fixture(autouse=True)

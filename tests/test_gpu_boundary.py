@@ -364,6 +364,33 @@ def test_staged_decode_step_agrees_with_the_row_major_fused_step(monkeypatch):
 
 
 @pytest.mark.gpu
+def test_greedy_token_from_the_head_launch_equals_argmax_over_logits(monkeypatch):
+    """decode_one_token on an int4 model: the head launch that reduces its own columns picks the tokens that argmax over
+    the stored logits picks (FUSE_HEAD_ARGMAX off), eagerly and through the captured graph."""
+    import easy_to_hard_amd.model as model_mod
+
+    cfg = model_mod.ModelArgs.from_name("7B")  # two layers of the 7B shape: every launch of the step has a staged form
+    cfg.n_layer = 2
+    model = model_mod.random_quantized_transformer(cfg, "int4", 128, device=DEV, seed=11)
+    bsz = 32
+    with torch.no_grad():
+        model.setup_caches(max_batch_size=bsz, max_seq_length=64)
+        prompt = torch.randint(0, cfg.vocab_size, (bsz, 9), generator=torch.Generator().manual_seed(2)).to(DEV)
+        stepper = GraphedDecodeStep(model, bsz, DEV)  # (its capture warm-up writes cache row 0: the prompt comes after it)
+        cur = prefill(model, prompt, torch.arange(0, 9, device=DEV))
+        pos = torch.tensor([9], device=DEV, dtype=torch.int64)
+        assert model.staged_step_supported(bsz)
+        fused = decode_one_token(model, cur, pos)
+        graphed = stepper.step(cur, pos).clone()
+        monkeypatch.setattr(model_mod, "FUSE_HEAD_ARGMAX", False)
+        plain = decode_one_token(model, cur, pos)
+        logits = model(cur, pos)
+    assert fused.shape == (bsz, 1) and fused.dtype == torch.int64
+    assert torch.equal(fused, plain) and torch.equal(graphed, plain)
+    assert torch.equal(plain, torch.argmax(logits[:, -1].float(), dim=-1, keepdim=True))
+
+
+@pytest.mark.gpu
 def test_read_only_probe_accepts_and_rejects_as_declared():
     """e2h_stream_read_probe (the launch behind `bench.py --floor`): it writes nothing, so what can be checked is that
     the documented argument ranges are accepted (empty launch, private bytes only, private + shared) and that bad sizes,

@@ -195,3 +195,34 @@ def test_decode_attention_staged_equals_the_row_major_kernel(n_head, n_kv):
     out = ops.decode_attention(q, kc, vc, pos)
     xs = ops.decode_attention_staged(q, kc, vc, pos)
     _assert_staged_equal(xs, bf16_to_np(out.view(bsz, n_head * hd)), bsz)
+
+
+@pytest.mark.parametrize("g", [32, 64, 128])
+@pytest.mark.parametrize("shape", [(48, 512), (32000, 4096), (1000 * 16, 1024)])
+def test_staged_argmax_head_equals_argmax_over_the_stored_product(g, shape):
+    """The LM head launch that reduces its own columns (greedy token, no logits stored) against argmax_rows over the
+    product the plain epilogue stores: identical tokens for 1 .. 64 rows, including rows whose maximum is tied between
+    columns of different workgroups (lowest column wins) and a NaN (counts as the maximum)."""
+    n, k = shape
+    _, _, packed_d, sz_d = _case(n, k, g, seed=g + 3)
+    lin = _Lin(n, k, g, packed_d, sz_d)
+    for m in (1, 16, 32, 33, 64):
+        if not ops.int4_staged_supported(m, lin, ops.STAGED_ARGMAX):
+            continue
+        x = randn_bf16((m, k), seed=m + 7)
+        if m >= 16:
+            x[3] = 0.0                      # every logit of the row equals exactly 0: the tie goes to column 0
+            x[5, 0] = float("nan")          # a NaN activation makes every logit of the row NaN: column 0 as well
+        xs = ops.stage_x(x.to(DEV))
+        want = ops.argmax_rows(ops.int4_mm_staged(xs, packed_d, g, sz_d))
+        got = ops.int4_mm_staged_argmax(xs, packed_d, g, sz_d)
+        assert got.dtype == torch.int64 and got.shape == (m, 1)
+        assert torch.equal(got, want), (m, (got != want).nonzero().tolist())
+        if m >= 16:
+            assert got[3, 0].item() == 0 and got[5, 0].item() == 0
+
+
+def test_staged_argmax_head_is_covered_for_the_benchmark_heads():
+    # the 7B head at 32 rows and the 34B head (group size 64) at 64 rows: the configurations the decode benchmark runs
+    for rows, n, k, g in ((32, 32000, 4096, 128), (64, 32000, 8192, 64)):
+        assert ops._lib.load().e2h_int4_mm_staged_supported(rows, n, k, g, ops.STAGED_ARGMAX) == 1
