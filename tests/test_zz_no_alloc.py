@@ -61,3 +61,49 @@ def test_static_scratch_entry_point_rejects_what_exceeds_its_buffer():
     assert rc == -9 and "scratch" in _lib.status_string(rc)
     rc = lib.e2h_int4_mm_static_scratch(None, ops._ptr(packed), ops._ptr(sz), ops._ptr(y), 4, 64, 256, g, 8, ops._stream(x))
     assert rc == -1
+
+
+def test_static_scratch_entry_point_leaves_device_memory_as_it_found_it_and_replays_from_a_graph():
+    """What the entry point is for: a warmed call changes neither the free device memory nor needs anything a HIP graph
+    capture forbids; replays of the captured call, with eager work between them, give the eager result every time."""
+    lib = _lib.load()
+    g = 128
+    w = randn_bf16((4096, 4096), std=0.02, seed=41).to(DEV)
+    packed, sz = e2h.prepare_int4_weight_and_scales_and_zeros(w, g, 8)
+    x = randn_bf16((32, 4096), seed=42).to(DEV)
+    y = torch.empty((32, 4096), dtype=torch.bfloat16, device=DEV)
+
+    def call():
+        rc = lib.e2h_int4_mm_static_scratch(ops._ptr(x), ops._ptr(packed), ops._ptr(sz), ops._ptr(y), 32, 4096, 4096, g, 8, ops._stream(x))
+        _lib.check(rc, "e2h_int4_mm_static_scratch")
+
+    call()  # resolves the buffer's address on this device
+    torch.cuda.synchronize()
+    eager = y.clone()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    assert torch.equal(y, eager)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        call()
+    for i in range(4):
+        y.fill_(float("nan"))
+        # eager work on the shared scratch between the replays
+        x2 = randn_bf16((7, 4096), seed=50 + i).to(DEV)
+        y2 = torch.empty((7, 4096), dtype=torch.bfloat16, device=DEV)
+        rc = lib.e2h_int4_mm_static_scratch(ops._ptr(x2), ops._ptr(packed), ops._ptr(sz), ops._ptr(y2), 7, 4096, 4096, g, 8, ops._stream(x2))
+        _lib.check(rc, "e2h_int4_mm_static_scratch")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {i}"
