@@ -5,9 +5,10 @@
 //
 // Dequantize-to-bfloat16 form: every weight becomes a bfloat16 value w = bf16( fma(128 + q, s, fma(-136, s, z)) ) on its
 // way into the matrix cores (two float32 FMAs: the constant z - 136 s is rounded to float32 once per group, then one FMA
-// per weight, then round to nearest even; within one bfloat16 ulp of the single-rounded bf16(s * (q - 8) + z) and equal
-// to it whenever z - 136 s is exact in float32), and the products accumulate in float32 -- the arithmetic of the
-// kernel the reference calls, up to that ulp.  With 256 accumulator registers per lane there is no
+// per weight, then round to nearest even.  Against the single-rounded bf16(s * (q - 8) + z) this is off by at most
+// 2^-22 (|z| + 136 |s|) in front of the last rounding: the same bfloat16 value except at near-ties of that rounding
+// (one ulp then) and for weights that nearly cancel, |w| << |z - 136 s|), and the products accumulate in float32 -- the
+// arithmetic of the kernel the reference calls, up to that difference.  With 256 accumulator registers per lane there is no
 // room for per-group partial sums, and none are needed this way: no pass over x for group sums, no accumulator
 // prologue, no scaling of accumulators inside the loop.
 //

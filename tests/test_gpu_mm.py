@@ -538,6 +538,63 @@ def test_int4_gemm128_with_weights_that_dequantize_exactly():
     assert torch.equal(got.cpu(), want)
 
 
+def _two_fma_weights(codes, sz, g):
+    """The dequantizing kernel's conversion restated in numpy: c = float32(z - 136 s), w = bf16(float32((128 + q) s + c)).
+    Each float32 FMA is formed in float64 (exact for bfloat16 s, z of these magnitudes: products of two 8-bit
+    significands, sums whose exponents lie within 2^29 of each other) and rounded once to float32."""
+    s = np.repeat(sz[..., 0].astype(np.float64).T, g, axis=1)  # [n, k]
+    z = np.repeat(sz[..., 1].astype(np.float64).T, g, axis=1)
+    c = (z - 136.0 * s).astype(np.float32)
+    w = ((128.0 + codes.astype(np.float64)) * s + c.astype(np.float64)).astype(np.float32)
+    return qo.bf16_round(w), c
+
+
+@pytest.mark.parametrize("g", [32, 64, 128])
+def test_int4_gemm128_converted_weights_read_back_through_identity_activations(g):
+    """x = identity makes y[m][n] the kernel's own bfloat16 weight (one product 1 * w, every other term zero).  With
+    random bfloat16 (scale, zero) pairs -- not the benign ones a quantizer emits -- the weights must equal the two-FMA
+    conversion bit for bit, lie within one bfloat16 ulp of the single-rounded bf16(s (q - 8) + z), and equal it
+    wherever z - 136 s is a float32 value."""
+    n, k = 264, 256
+    gen = torch.Generator().manual_seed(77 + g)
+    codes = torch.randint(0, 16, (n, k), generator=gen, dtype=torch.int32)
+    scales = (torch.rand((k // g, n), generator=gen) * 0.02 + 1e-4).to(torch.bfloat16)
+    zeros = (torch.randn((k // g, n), generator=gen) * 0.05).to(torch.bfloat16)
+    sz = torch.stack([scales, zeros], dim=-1)
+    x = torch.eye(k, dtype=torch.bfloat16)
+    packed_d = ops.int4_pack(codes.to(DEV), 8)
+    _lib.set_option("int4_gemm_tile", 256)
+    try:
+        got = ops.int4_mm_direct(x.to(DEV), packed_d, g, sz.to(DEV))
+    finally:
+        _lib.set_option("int4_gemm_tile", 0)
+    got = bf16_to_np(got.cpu()).T.astype(np.float64)  # [n, k]
+    want, c = _two_fma_weights(codes.numpy(), bf16_to_np(sz), g)
+    assert np.array_equal(got, want.astype(np.float64))
+    s64 = np.repeat(bf16_to_np(sz)[..., 0].astype(np.float64).T, g, axis=1)
+    z64 = np.repeat(bf16_to_np(sz)[..., 1].astype(np.float64).T, g, axis=1)
+    exact = s64 * (codes.numpy().astype(np.float64) - 8.0) + z64  # exact in float64 at these magnitudes
+    single = _bf16_round_f64(exact)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(exact), 1e-300))) - 7)
+    c_mag = 136.0 * np.abs(s64) + np.abs(z64)
+    # half a bfloat16 ulp of the exact value from the final rounding, and the two float32 roundings (of z - 136 s, of
+    # the FMA's result) in front of it, each at most 2^-24 of a value no larger than |z| + 136 |s| + 143 |s|
+    assert np.all(np.abs(got - exact) <= 0.5 * ulp + 2.0 ** -22 * c_mag)
+    differs = got != single
+    assert differs.mean() < 0.01  # near-ties of the last rounding and nearly cancelling weights only
+    ordinary = np.abs(exact) >= 2.0 ** -6 * c_mag
+    assert np.all(np.abs(got - single)[ordinary] <= ulp[ordinary] * (1 + 2.0 ** -7))
+
+
+def _bf16_round_f64(x):
+    """float64 -> nearest bfloat16 value (ties to even), as float64, in one rounding (normal magnitudes only)."""
+    u = np.ascontiguousarray(x, dtype=np.float64).view(np.uint64)
+    drop = np.uint64(52 - 7)
+    lsb = (u >> drop) & np.uint64(1)
+    r = ((u + ((np.uint64(1) << (drop - np.uint64(1))) - np.uint64(1)) + lsb) >> drop) << drop
+    return r.view(np.float64)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["int8", "int4"])
 def test_many_row_kernels_with_an_output_that_is_only_2_byte_aligned(mode):
